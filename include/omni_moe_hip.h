@@ -1,0 +1,203 @@
+/*
+ * omni_moe_hip.h -- C ABI of libomni_moe_hip.so: the gfx950 (MI355X) operator set
+ * behind omni-infer's W8A8 dynamic-quant fused-MoE layer.
+ *
+ * The reference reaches its device arithmetic through `torch_npu.npu_*` Python
+ * operators (closed CANN kernels).  Each entry point below replaces one such
+ * operator family; the reference call sites are cited per function (paths are
+ * relative to the reference tree).  All pointers are device pointers unless
+ * stated, all sizes are explicit, `stream` is a hipStream_t passed as void*.
+ *
+ * Conventions
+ *  - every function returns 0 on success and a negative OMNI_E_* code on a
+ *    rejected argument; omni_moe_last_error() then describes it (thread local);
+ *  - nothing here allocates device memory, synchronises the device or copies to
+ *    the host: all work is enqueued on `stream`, data dependent sizes (rows per
+ *    expert) stay in device memory, so a call sequence can be captured in a HIP
+ *    graph;
+ *  - the library keeps no device state between calls.
+ *
+ * Packed weight layout ("frag16"), produced by omni_moe_pack_weight
+ *  A logical matrix B[Kdim][N] (Kdim = reduction dim, N = output channels) is
+ *  stored as tiles of 16 output channels x 64 reduction elements, 1024 bytes each:
+ *      offset(k, n) = (((n/16) * (Kdim/64) + k/64) * 64 + (n%16) + 16*((k%64)/16)) * 16 + k%16
+ *  so that lane l of a wavefront reads its 16-byte operand of
+ *  v_mfma_i32_16x16x64_i8 at tile_base + 16*l, and a 16-channel strip is
+ *  contiguous along k.  Requires Kdim % 64 == 0 and N % 16 == 0.
+ */
+#ifndef OMNI_MOE_HIP_H
+#define OMNI_MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OMNI_OK 0
+#define OMNI_E_INVALID (-1)      /* null pointer, negative size, inconsistent arguments */
+#define OMNI_E_UNSUPPORTED (-2)  /* shape outside what the kernels are built for */
+#define OMNI_E_WORKSPACE (-3)    /* workspace too small */
+#define OMNI_E_LAUNCH (-4)       /* the HIP runtime refused a launch */
+
+/* dtype codes of activations / row buffers */
+#define OMNI_DT_BF16 0
+#define OMNI_DT_F32 1
+#define OMNI_DT_F16 2
+
+/* omni_moe_route: score_fn */
+#define OMNI_SCORE_SOFTMAX 0
+#define OMNI_SCORE_SIGMOID 1
+/* omni_moe_route: group_mode */
+#define OMNI_GROUP_MAX 0
+#define OMNI_GROUP_TOP2SUM 1
+
+/* gemm flags */
+#define OMNI_GEMM1_BF16_INTERMEDIATE 1 /* round the dequantised gate/up and the SwiGLU product to bf16
+                                          (numerics of the non-EP pipeline, compressed_tensors_moe.py:242-247) */
+/* combine: how src_to_dst is indexed */
+#define OMNI_IDX_TOKEN_MAJOR 0 /* n*K + k  (npu_moe_init_routing_v2 row_idx_type=1; finalize drop_pad_mode=2) */
+#define OMNI_IDX_K_MAJOR 1     /* k*T + n  (npu_moe_init_routing; finalize drop_pad_mode=0) */
+/* combine: order in which a token's rows are added */
+#define OMNI_ORDER_SLOT 0 /* ascending sorted slot  (npu_grouped_matmul_finalize_routing) */
+#define OMNI_ORDER_K 1    /* ascending k            (npu_moe_finalize_routing) */
+
+/* Last error message of the calling thread ("" if none). */
+const char* omni_moe_last_error(void);
+/* ABI version of this header (bumped on incompatible change). */
+int omni_moe_abi_version(void);
+
+/*
+ * Router.  Replaces torch_npu.npu_moe_gating_top_k
+ * (omni/models/common/layers/moe/fused_moe/layer.py:341-351), the torch
+ * grouped_topk (omni/models/common/layers/moe/fused_moe/fused_moe.py:38-84) and
+ * torch_npu.npu_moe_gating_top_k_softmax (fused_moe.py:29).
+ *   logits [T,E] fp32, bias [E] fp32 or NULL.
+ *   score s = softmax(logits) or sigmoid(logits); c = s + bias.
+ *   n_group > 1: group score = max c (GROUP_MAX) or sum of the two largest c
+ *   (GROUP_TOP2SUM); the topk_group best groups are kept; other experts take part
+ *   with score -inf (masked_fill_zero = 0) or 0.0 (masked_fill_zero = 1).
+ *   top-K by c, descending, ties to the lower id.
+ *   weight = s[id] (weight_from_c = 0) or the selection score (weight_from_c = 1);
+ *   renorm != 0: weight /= (sum of the K weights in output order + eps);
+ *   weight *= scale.
+ * Outputs topk_w [T,K] fp32, topk_ids [T,K] int32.  E <= 512, K <= 64, n_group <= 64.
+ */
+int omni_moe_route(const float* logits, const float* bias, int T, int E, int n_group, int topk_group, int K,
+                   int score_fn, int group_mode, int masked_fill_zero, int weight_from_c, int renorm, float scale,
+                   float eps, float* topk_w, int32_t* topk_ids, void* stream);
+
+/*
+ * Per-row dynamic int8 quantisation.  Replaces torch_npu.npu_dynamic_quant
+ * (omni/models/common/layers/moe/deepseek_moe.py:247,323,612;
+ * omni/quantization/compressed_tensors/compressed_tensors_moe.py:241,247;
+ * fused_moe.py:668; schemes/compressed_tensors_w8a8_int8.py:97).
+ *   x [rows, cols] of in_dtype with row stride ld (elements);
+ *   scale[r] = max|x[r,:]| / 127; q = clamp(rint(x / scale), -128, 127); a zero row gives 0, 0.
+ */
+int omni_dynamic_quant(const void* x, int in_dtype, int64_t rows, int cols, int64_t ld, int8_t* q, float* scale,
+                       void* stream);
+
+/*
+ * Sort (token, k) assignments by expert.  Replaces torch_npu.npu_moe_init_routing +
+ * npu_moe_compute_expert_tokens (compressed_tensors_moe.py:235-237) and
+ * npu_moe_init_routing_v2 with active_expert_range (fused_moe.py:514-515, :607-618).
+ *   topk_ids [T,K] int32; entries with lo <= id < hi are kept.
+ *   idx_mode selects how an assignment is numbered ("source index"): n*K+k or k*T+n.
+ *   Stable by expert id; inside an expert ascending n*K+k.
+ *   sorted_src [T*K]: source index of every sorted slot (dropped assignments follow the kept
+ *   ones, in their original order); src_to_dst [T*K]: slot of every source index, -1 if dropped;
+ *   counts [hi-lo]; offsets [hi-lo+1] (exclusive prefix, offsets[hi-lo] = kept total).
+ *   workspace: omni_moe_permute_workspace_bytes(T, K, hi-lo).
+ */
+int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode, int32_t* sorted_src,
+                     int32_t* src_to_dst, int32_t* counts, int32_t* offsets, void* workspace, size_t ws_bytes,
+                     void* stream);
+size_t omni_moe_permute_workspace_bytes(int T, int K, int n_local);
+
+/*
+ * Materialise the sorted rows (the expanded_x / dynamic_quant_scale outputs of
+ * npu_moe_init_routing(_v2), fused_moe.py:514-515).  row m < offsets[n_local] is a copy of
+ * source row token(sorted_src[m]); elem_bytes is the byte size of a row element.
+ */
+int omni_moe_gather_rows(const void* x, int elem_bytes, int H, const float* x_scale, const int32_t* sorted_src,
+                         const int32_t* offsets, int n_local, int T, int K, int idx_mode, void* rows_out,
+                         float* scale_out, void* stream);
+
+/*
+ * One-off weight re-layout into the frag16 format (the analogue of
+ * torch_npu.npu_format_cast(w, 29), compressed_tensors_moe.py:97-99).
+ *   src_layout 0: w is [G, Kdim, N] (after process_weights_after_loading's transpose,
+ *   compressed_tensors_moe.py:95-96); 1: w is [G, N, Kdim] (as create_weights declares it, :44-60).
+ */
+int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N, int8_t* packed, void* stream);
+
+/*
+ * GEMM1 + dequant + SwiGLU + per-row requant.  Replaces
+ * npu_grouped_matmul(output_dtype=int32) + npu_dequant_swiglu_quant
+ * (fused_moe.py:531-534, :552-561, :670-677; deepseek_moe.py:465-471; activation.py:15-27),
+ * and with OMNI_GEMM1_BF16_INTERMEDIATE npu_grouped_matmul(bf16) + npu_swiglu + npu_dynamic_quant
+ * (compressed_tensors_moe.py:242-247).
+ *   Rows are grouped: group g owns rows [offsets[g], offsets[g+1]); an optional extra group
+ *   (w13_extra != NULL) owns rows [offsets[G], offsets[G] + extra_rows) and maps row r to source
+ *   row r - offsets[G] (the shared expert on every token).
+ *   Row m of a regular group reads x_q[sorted_src[m] / src_div] (idx_mode TOKEN_MAJOR) or
+ *   x_q[sorted_src[m] % src_mod] (K_MAJOR); sorted_src NULL: row m reads x_q[m].
+ *   acc = x_q[row] . W13[g]  (int32, exact);  d = (float(acc) * w13_scale[g][n]) * x_scale[row];
+ *   y = silu(d[:I]) * d[I:];  h_scale[m] = max|y| / 127;  h_q = rint(y / h_scale).
+ *   w13 packed: G matrices of Kdim = H, N = 2I (gate channels first).
+ *   acc_dbg (nullable) [M_cap, 2I] receives the int32 accumulators.
+ *   workspace: omni_moe_gemm1_workspace_bytes(M_cap, I).
+ */
+int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode,
+                                int T, int K, const int8_t* w13_packed, const float* w13_scale,
+                                const int8_t* w13_extra, const float* w13_extra_scale, int extra_rows,
+                                const int32_t* offsets, int G, int H, int I, int64_t M_cap, int flags, int8_t* h_q,
+                                float* h_scale, int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream);
+size_t omni_moe_gemm1_workspace_bytes(int64_t M_cap, int I);
+
+/*
+ * GEMM2 + dequant.  Replaces npu_grouped_matmul(scale=, per_token_scale=, output_dtype=bf16)
+ * (fused_moe.py:570-574, :681-685; deepseek_moe.py:473-477; compressed_tensors_moe.py:249-251)
+ * and npu_quant_matmul(pertoken_scale=) (schemes/compressed_tensors_w8a8_int8.py:105-109).
+ *   rows_out[m, :] = cast((float(h_q[m] . W2[g]) * w2_scale[g][:]) * h_scale[m]), out_dtype BF16 or F32.
+ *   w2 packed: G matrices of Kdim = I, N = H.  Grouping as in GEMM1.
+ */
+int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
+                           const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows,
+                           const int32_t* offsets, int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out,
+                           int32_t* acc_dbg, void* stream);
+
+/*
+ * Weighted un-permute.  Replaces the routing half of npu_grouped_matmul_finalize_routing
+ * (fused_moe.py:536), npu_moe_finalize_routing (compressed_tensors_moe.py:253;
+ * deepseek_moe.py:292-301) and the shared-expert add (deepseek_moe.py:303,366).
+ *   acc = init ? float(init[n]) : 0;  for each kept assignment of token n, in `order`:
+ *   acc += topk_w[n,k] * float(rows[src_to_dst[idx(n,k)]]);  out = bf16(acc);
+ *   if post_add != NULL: out = bf16(float(out) + float(bf16(post_add_row n)))   (post_add has rows_dtype,
+ *   row n of it is added; pass rows + offsets_total*H to add the extra group's rows).
+ */
+int omni_moe_combine(const void* rows, int rows_dtype, const float* topk_w, const int32_t* src_to_dst, int idx_mode,
+                     int order, int T, int K, int H, const void* init_bf16, const void* post_add,
+                     const int32_t* post_add_row0, void* out_bf16, void* stream);
+
+/*
+ * The whole layer in one call: quant (if x is bf16) -> permute -> GEMM1 epilogue -> GEMM2 -> combine,
+ * the sequence of fused_experts_w8a8_allgather_ep (fused_moe.py:489-538) with the shared expert
+ * (deepseek_moe.py:64-118,244,303) carried as an extra group.  Routing weights and ids are inputs
+ * (omni_moe_route makes them).  x_dtype BF16: x is quantised first; x_dtype -1: x is int8 and
+ * x_scale is given.  Returns bf16 [T,H].
+ */
+int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
+                        const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
+                        const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
+                        const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
+                        const float* sh2_scale, int H, int I, void* out_bf16, void* workspace, size_t ws_bytes,
+                        void* stream);
+size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OMNI_MOE_HIP_H */

@@ -1,0 +1,227 @@
+// Weighted un-permute (finalize routing), the library's error state and the whole-layer entry.
+//
+// combine: grid (token, column chunk of 1024).  The block first lists the token's kept
+// assignments (slot, weight) in LDS, ordered by slot or by k as asked, then every thread
+// accumulates four consecutive columns in fp32, one multiply and one add per row, in that order.
+#include "common.h"
+
+#include <string.h>
+
+// ---------------------------------------------------------------- error state
+static thread_local char g_err[512] = "";
+void omni_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+extern "C" const char* omni_moe_last_error(void) { return g_err; }
+extern "C" int omni_moe_abi_version(void) { return 1; }
+
+namespace {
+
+constexpr int KMAX = 64;
+
+struct CombineArgs {
+  const void* rows;
+  int rows_dtype;
+  const float* topk_w;
+  const int32_t* src_to_dst;
+  int idx_mode, order, T, K, H;
+  const uint16_t* init;
+  const void* post_add;
+  const int32_t* post_add_row0;
+  uint16_t* out;
+};
+
+template <int DT>
+__device__ __forceinline__ void load4(const void* base, size_t row, int H, int c, int ncol, float* v) {
+  if constexpr (DT == OMNI_DT_F32) {
+    const float* p = (const float*)base + row * H + c;
+    if (ncol == 4) {
+      v4f t = *(const v4f*)p;
+      v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+    } else {
+      for (int j = 0; j < 4; ++j) v[j] = j < ncol ? p[j] : 0.0f;
+    }
+  } else {
+    const uint16_t* p = (const uint16_t*)base + row * H + c;
+    if (ncol == 4) {
+      v2i t = *(const v2i*)p;
+      v[0] = bf16_to_f32((uint16_t)((uint32_t)t[0] & 0xffffu));
+      v[1] = bf16_to_f32((uint16_t)((uint32_t)t[0] >> 16));
+      v[2] = bf16_to_f32((uint16_t)((uint32_t)t[1] & 0xffffu));
+      v[3] = bf16_to_f32((uint16_t)((uint32_t)t[1] >> 16));
+    } else {
+      for (int j = 0; j < 4; ++j) v[j] = j < ncol ? bf16_to_f32(p[j]) : 0.0f;
+    }
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
+  __shared__ int s_slot[KMAX];
+  __shared__ float s_w[KMAX];
+  __shared__ int s_cnt;
+  const int n = blockIdx.x;
+  if (threadIdx.x == 0) {
+    int cnt = 0;
+    for (int k = 0; k < a.K; ++k) {
+      int idx = (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? n * a.K + k : k * a.T + n;
+      int slot = a.src_to_dst[idx];
+      if (slot < 0) continue;
+      float wv = a.topk_w[(size_t)n * a.K + k];
+      int pos = cnt;
+      if (a.order == OMNI_ORDER_SLOT) {  // insertion by slot; k order otherwise
+        while (pos > 0 && s_slot[pos - 1] > slot) {
+          s_slot[pos] = s_slot[pos - 1];
+          s_w[pos] = s_w[pos - 1];
+          --pos;
+        }
+      }
+      s_slot[pos] = slot;
+      s_w[pos] = wv;
+      ++cnt;
+    }
+    s_cnt = cnt;
+  }
+  __syncthreads();
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c >= a.H) return;
+  const int ncol = min(4, a.H - c);
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (a.init) load4<OMNI_DT_BF16>(a.init, (size_t)n, a.H, c, ncol, acc);
+  const int cnt = s_cnt;
+  for (int j = 0; j < cnt; ++j) {
+    float v[4];
+    load4<DT>(a.rows, (size_t)s_slot[j], a.H, c, ncol, v);
+    const float wv = s_w[j];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float prod = wv * v[i];
+      acc[i] = acc[i] + prod;
+    }
+  }
+  uint16_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(acc[i]);
+  if (a.post_add) {
+    float v[4];
+    size_t r = (size_t)n + (a.post_add_row0 ? (size_t)*a.post_add_row0 : 0);
+    load4<DT>(a.post_add, r, a.H, c, ncol, v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(bf16_to_f32(o[i]) + round_bf16(v[i]));
+  }
+  uint16_t* op = a.out + (size_t)n * a.H + c;
+  if (ncol == 4) {
+    v2i t = {(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
+    *(v2i*)op = t;
+  } else {
+    for (int j = 0; j < ncol; ++j) op[j] = o[j];
+  }
+}
+
+inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+}  // namespace
+
+extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* topk_w, const int32_t* src_to_dst,
+                                int idx_mode, int order, int T, int K, int H, const void* init_bf16,
+                                const void* post_add, const int32_t* post_add_row0, void* out_bf16, void* stream) {
+  if (T < 0 || K <= 0 || H <= 0) OMNI_FAIL(OMNI_E_INVALID, "combine: bad sizes T=%d K=%d H=%d", T, K, H);
+  if (T == 0) return OMNI_OK;
+  if (K > KMAX) OMNI_FAIL(OMNI_E_UNSUPPORTED, "combine: K=%d > %d", K, KMAX);
+  if (!rows || !topk_w || !src_to_dst || !out_bf16) OMNI_FAIL(OMNI_E_INVALID, "combine: null pointer");
+  if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "combine: rows_dtype %d", rows_dtype);
+  if (H % 4 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "combine: H=%d must be a multiple of 4", H);
+  if (((uintptr_t)rows % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)init_bf16 % 8) || ((uintptr_t)post_add % 16))
+    OMNI_FAIL(OMNI_E_INVALID, "combine: misaligned pointer");
+  CombineArgs a{rows, rows_dtype, topk_w, src_to_dst, idx_mode, order, T, K, H, (const uint16_t*)init_bf16, post_add,
+                post_add_row0, (uint16_t*)out_bf16};
+  dim3 grid((unsigned)T, (unsigned)((H + 1023) / 1024)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (rows_dtype == OMNI_DT_F32) hipLaunchKernelGGL(combine_kernel<OMNI_DT_F32>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(combine_kernel<OMNI_DT_BF16>, grid, block, 0, st, a);
+  OMNI_CHECK_LAUNCH("combine");
+  return OMNI_OK;
+}
+
+// ---------------------------------------------------------------- whole layer
+namespace {
+struct LayerWs {
+  size_t x_q, x_s, sorted_src, src_to_dst, counts, offsets, perm_ws, h_q, h_s, g1_ws, rows, total;
+  size_t perm_bytes, g1_bytes;
+  int64_t M_cap;
+};
+LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
+  LayerWs L{};
+  L.M_cap = (int64_t)T * K + (with_shared ? T : 0);
+  size_t o = 0;
+  auto take = [&](size_t bytes) { size_t at = o; o += align256(bytes); return at; };
+  L.x_q = take((size_t)T * H);
+  L.x_s = take((size_t)T * 4);
+  L.sorted_src = take((size_t)T * K * 4);
+  L.src_to_dst = take((size_t)T * K * 4);
+  L.counts = take((size_t)G * 4);
+  L.offsets = take((size_t)(G + 1) * 4);
+  L.perm_bytes = omni_moe_permute_workspace_bytes(T, K, G);
+  L.perm_ws = take(L.perm_bytes);
+  L.h_q = take((size_t)L.M_cap * I);
+  L.h_s = take((size_t)L.M_cap * 4);
+  L.g1_bytes = omni_moe_gemm1_workspace_bytes(L.M_cap, I);
+  L.g1_ws = take(L.g1_bytes);
+  L.rows = take((size_t)L.M_cap * H * 4);
+  L.total = o;
+  return L;
+}
+}  // namespace
+
+extern "C" size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared) {
+  if (T < 0 || K <= 0 || n_local <= 0 || H <= 0 || I <= 0) return 0;
+  return layer_layout(T, K, n_local, H, I, with_shared).total;
+}
+
+extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
+                                   const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
+                                   const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
+                                   const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
+                                   const float* sh2_scale, int H, int I, void* out_bf16, void* workspace,
+                                   size_t ws_bytes, void* stream) {
+  if (T < 0 || K <= 0 || hi <= lo || H <= 0 || I <= 0) OMNI_FAIL(OMNI_E_INVALID, "layer: bad sizes");
+  if (T == 0) return OMNI_OK;
+  if (!x || !topk_w || !topk_ids || !out_bf16 || !workspace) OMNI_FAIL(OMNI_E_INVALID, "layer: null pointer");
+  if (x_dtype == -1 && !x_scale_in) OMNI_FAIL(OMNI_E_INVALID, "layer: int8 input without scales");
+  const int G = hi - lo;
+  const int with_shared = sh13_packed != nullptr;
+  if (with_shared && (!sh13_scale || !sh2_packed || !sh2_scale)) OMNI_FAIL(OMNI_E_INVALID, "layer: incomplete shared expert");
+  if ((uintptr_t)workspace % 256) OMNI_FAIL(OMNI_E_INVALID, "layer: workspace must be 256-byte aligned");
+  LayerWs L = layer_layout(T, K, G, H, I, with_shared);
+  if (ws_bytes < L.total) OMNI_FAIL(OMNI_E_WORKSPACE, "layer: workspace %zu < %zu", ws_bytes, L.total);
+  char* ws = (char*)workspace;
+  const int8_t* xq = (const int8_t*)x;
+  const float* xs = x_scale_in;
+  int rc;
+  if (x_dtype != -1) {
+    rc = omni_dynamic_quant(x, x_dtype, T, H, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), stream);
+    if (rc) return rc;
+    xq = (const int8_t*)(ws + L.x_q);
+    xs = (const float*)(ws + L.x_s);
+  }
+  int32_t* sorted_src = (int32_t*)(ws + L.sorted_src);
+  int32_t* src_to_dst = (int32_t*)(ws + L.src_to_dst);
+  int32_t* offsets = (int32_t*)(ws + L.offsets);
+  rc = omni_moe_permute(topk_ids, T, K, lo, hi, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts),
+                        offsets, ws + L.perm_ws, L.perm_bytes, stream);
+  if (rc) return rc;
+  const int extra = with_shared ? T : 0;
+  rc = omni_moe_gemm1_swiglu_quant(xq, xs, sorted_src, OMNI_IDX_TOKEN_MAJOR, T, K, w13_packed, w13_scale, sh13_packed,
+                                   sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),
+                                   (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, stream);
+  if (rc) return rc;
+  rc = omni_moe_gemm2_dequant((const int8_t*)(ws + L.h_q), (const float*)(ws + L.h_s), w2_packed, w2_scale, sh2_packed,
+                              sh2_scale, extra, offsets, G, H, I, L.M_cap, OMNI_DT_F32, ws + L.rows, nullptr, stream);
+  if (rc) return rc;
+  return omni_moe_combine(ws + L.rows, OMNI_DT_F32, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
+                          nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,
+                          stream);
+}

@@ -1,0 +1,209 @@
+// Shared device helpers for the gfx950 MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/omni_moe_hip.h"
+
+// Every floating-point operation below is meant to round once: no contraction into FMA.
+#pragma clang fp contract(off)
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+#define WAVE 64
+
+// ---------------------------------------------------------------- host side error state
+void omni_set_error(const char* fmt, ...);
+#define OMNI_FAIL(code, ...)        \
+  do {                              \
+    omni_set_error(__VA_ARGS__);    \
+    return (code);                  \
+  } while (0)
+#define OMNI_CHECK_LAUNCH(what)                                                            \
+  do {                                                                                     \
+    hipError_t e__ = hipGetLastError();                                                    \
+    if (e__ != hipSuccess) OMNI_FAIL(OMNI_E_LAUNCH, "%s: %s", what, hipGetErrorString(e__)); \
+  } while (0)
+
+// ---------------------------------------------------------------- specified transcendental
+// exp with a fixed operation sequence: clamp to [-87, 87], Cody-Waite reduction by ln2 split in
+// two constants, the Cephes expf polynomial by Horner, scaling by 2^n through the exponent field.
+// One rounding per operation (this file is compiled with contraction off).
+__device__ __forceinline__ float exp_spec(float x) {
+  x = fminf(fmaxf(x, -87.0f), 87.0f);
+  float n = rintf(x * 1.44269504088896341f);
+  float r = x - n * 0.693359375f;
+  r = r - n * -2.12194440e-4f;
+  float p = 1.9875691500e-4f;
+  p = p * r;
+  p = p + 1.3981999507e-3f;
+  p = p * r;
+  p = p + 8.3334519073e-3f;
+  p = p * r;
+  p = p + 4.1665795894e-2f;
+  p = p * r;
+  p = p + 1.6666665459e-1f;
+  p = p * r;
+  p = p + 5.0000001201e-1f;
+  float y = p * (r * r);
+  y = y + r;
+  y = y + 1.0f;
+  int ni = (int)n;
+  return y * __int_as_float((ni + 127) << 23);
+}
+__device__ __forceinline__ float sigmoid_spec(float x) { return 1.0f / (1.0f + exp_spec(-x)); }
+__device__ __forceinline__ float silu_spec(float x) { return x / (1.0f + exp_spec(-x)); }
+
+// ---------------------------------------------------------------- bf16 <-> fp32
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+__device__ __forceinline__ float f16_to_f32(uint16_t h) {
+  _Float16 v;
+  __builtin_memcpy(&v, &h, 2);
+  return (float)v;
+}
+
+// ---------------------------------------------------------------- cross-lane exchange
+// DPP inside a row of 16 lanes, ds_bpermute across rows.  xchg<S>(v) returns the value held by
+// the partner lane of a butterfly step over 2*S lanes; every lane of a 2*S cluster that already
+// agrees on a cluster value receives the other half's value, which is all an all-reduce needs.
+template <int S>
+__device__ __forceinline__ int xchg_i(int v) {
+  if constexpr (S == 1) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false);       // quad_perm [1,0,3,2]
+  else if constexpr (S == 2) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false);  // quad_perm [2,3,0,1]
+  else if constexpr (S == 4) return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, false); // row_half_mirror
+  else if constexpr (S == 8) return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false); // row_mirror
+  else return __shfl_xor(v, S, WAVE);
+}
+template <int S>
+__device__ __forceinline__ float xchg_f(float v) { return __int_as_float(xchg_i<S>(__float_as_int(v))); }
+template <int S>
+__device__ __forceinline__ uint64_t xchg_u64(uint64_t v) {
+  uint32_t lo = (uint32_t)xchg_i<S>((int)(uint32_t)v);
+  uint32_t hi = (uint32_t)xchg_i<S>((int)(uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ float wave_allmax_f(float v) {
+  v = fmaxf(v, xchg_f<1>(v));
+  v = fmaxf(v, xchg_f<2>(v));
+  v = fmaxf(v, xchg_f<4>(v));
+  v = fmaxf(v, xchg_f<8>(v));
+  v = fmaxf(v, xchg_f<16>(v));
+  v = fmaxf(v, xchg_f<32>(v));
+  return v;
+}
+// butterfly sum, pairing order 1,2,4,8,16,32 (the order the checker states)
+__device__ __forceinline__ float wave_allsum_f(float v) {
+  v = v + xchg_f<1>(v);
+  v = v + xchg_f<2>(v);
+  v = v + xchg_f<4>(v);
+  v = v + xchg_f<8>(v);
+  v = v + xchg_f<16>(v);
+  v = v + xchg_f<32>(v);
+  return v;
+}
+__device__ __forceinline__ uint64_t wave_allmax_u64(uint64_t v) {
+  uint64_t o;
+  o = xchg_u64<1>(v); v = o > v ? o : v;
+  o = xchg_u64<2>(v); v = o > v ? o : v;
+  o = xchg_u64<4>(v); v = o > v ? o : v;
+  o = xchg_u64<8>(v); v = o > v ? o : v;
+  o = xchg_u64<16>(v); v = o > v ? o : v;
+  o = xchg_u64<32>(v); v = o > v ? o : v;
+  return v;
+}
+// max over the 16 lanes of a DPP row
+__device__ __forceinline__ float row16_allmax_f(float v) {
+  v = fmaxf(v, xchg_f<1>(v));
+  v = fmaxf(v, xchg_f<2>(v));
+  v = fmaxf(v, xchg_f<4>(v));
+  v = fmaxf(v, xchg_f<8>(v));
+  return v;
+}
+__device__ __forceinline__ int wave_incl_scan_i(int v, int lane) {
+#pragma unroll
+  for (int s = 1; s < WAVE; s <<= 1) {
+    int o = __shfl_up(v, s, WAVE);
+    if (lane >= s) v += o;
+  }
+  return v;
+}
+
+// floats to unsigned keys with the same order
+__device__ __forceinline__ uint32_t f32_order_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// ---------------------------------------------------------------- quantisation of one value
+__device__ __forceinline__ int quant_i8(float x, float s) {
+  float q = rintf(x / s);
+  q = fminf(fmaxf(q, -128.0f), 127.0f);
+  return (int)q;
+}
+
+// ---------------------------------------------------------------- grouped row-block lookup
+// Row blocks of BM rows are numbered group by group (a group with c rows has ceil(c/BM) of them).
+// Finds the group and the first row of block `b`; returns false when b is past the last block.
+// offsets[0..G] is the exclusive prefix of the regular groups; an extra group of extra_rows rows
+// follows at offsets[G].  Every lane of the calling wave gets the same answer.
+struct RowBlock {
+  int group;
+  int row0;
+  int nrows;
+};
+__device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offsets, int G, int extra_rows, int BM,
+                                               int b, RowBlock& rb) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int Gt = G + (extra_rows > 0 ? 1 : 0);
+  const int per = (Gt + WAVE - 1) / WAVE;
+  const int g0 = lane * per;
+  int mine = 0;
+  for (int j = 0; j < per; ++j) {
+    int g = g0 + j;
+    if (g < Gt) {
+      int c = (g < G) ? (offsets[g + 1] - offsets[g]) : extra_rows;
+      mine += (c + BM - 1) / BM;
+    }
+  }
+  int incl = wave_incl_scan_i(mine, lane);
+  int excl = incl - mine;
+  int total = __shfl(incl, WAVE - 1, WAVE);
+  if (b >= total) return false;
+  uint64_t owner_mask = __ballot(b >= excl && b < incl);
+  int owner = __ffsll((unsigned long long)owner_mask) - 1;
+  int grp = -1, row0 = 0, nrows = 0;
+  if (lane == owner) {
+    int acc = excl;
+    for (int j = 0; j < per; ++j) {
+      int g = g0 + j;
+      if (g >= Gt) break;
+      int start = offsets[g < G ? g : G];
+      int c = (g < G) ? (offsets[g + 1] - start) : extra_rows;
+      int nb = (c + BM - 1) / BM;
+      if (b < acc + nb) {
+        grp = g;
+        row0 = start + (b - acc) * BM;
+        nrows = min(BM, c - (b - acc) * BM);
+        break;
+      }
+      acc += nb;
+    }
+  }
+  rb.group = __shfl(grp, owner, WAVE);
+  rb.row0 = __shfl(row0, owner, WAVE);
+  rb.nrows = __shfl(nrows, owner, WAVE);
+  return true;
+}

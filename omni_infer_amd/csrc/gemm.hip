@@ -1,0 +1,611 @@
+// Grouped int8 x int8 -> int32 GEMMs on v_mfma_i32_16x16x64_i8 with fused epilogues.
+//
+// Operand layouts
+//   B (weights) is in the frag16 format: tiles of 16 output channels x 64 reduction elements,
+//   1 KiB each, in exactly the order the MFMA wants them in registers (lane l owns bytes
+//   [16 l, 16 l + 16) of a tile).  A 16-channel strip is contiguous along k, so a wavefront that
+//   walks k streams one contiguous region per strip with 16-byte loads.
+//   A (int8 activations) is row major in memory.  It is staged through LDS in the same fragment
+//   order: one wavefront load instruction fetches a 16 row x 64 byte fragment (lane l: row l%16,
+//   bytes 16*(l/16)..+16) and stores it linearly, so LDS writes and the later ds_read_b128
+//   fragment reads are both conflict free.  The gather by sorted slot (the permutation of the
+//   MoE) happens in this load: no sorted copy of the activations is ever made.
+//   C: lane l of a 16x16 tile holds rows 4*(l/16)..+4 of column l%16.
+//
+// Two kernels share the epilogues:
+//   gemm_stream  rows per group <= 64 or so: weight streaming.  Each wavefront owns whole
+//                16-channel strips of B and loads them straight from global memory into MFMA
+//                registers through a ring of D outstanding k-steps (each weight byte is used by
+//                exactly one wavefront, so LDS staging would only add traffic); A is small and
+//                shared by the four wavefronts of a block through LDS.
+//   gemm_tile    large row counts: 256 x 128 block tiles, A and B both staged through LDS with
+//                register prefetch of the next k-step, each wavefront a 128 x 64 sub-tile.
+//
+// GEMM1 pairs gate channel n with up channel I + n in the same lane so SwiGLU needs no exchange.
+// Its epilogue writes y = silu(gate) * up in fp32 to a scratch matrix and folds max|y| of each
+// row into a per-row word with an atomic max on the float's bit pattern (exact and order
+// independent for non-negative floats); a second small kernel quantises the rows.
+#include "common.h"
+
+namespace {
+
+struct GemmArgs {
+  const int8_t* a_q;        // GEMM1: [T, Kdim] source rows; GEMM2: [M_cap, Kdim] sorted rows
+  const float* a_scale;     // per source row (GEMM1) / per sorted row (GEMM2)
+  const int32_t* sorted_src;  // GEMM1 only, nullable
+  int idx_mode, T, K;
+  const int8_t* w;
+  const float* w_scale;
+  const int8_t* w_extra;
+  const float* w_extra_scale;
+  int extra_rows;
+  const int32_t* offsets;
+  int G;
+  int Kdim;  // reduction length
+  int N;     // output channels of the GEMM: 2I (GEMM1) or H (GEMM2)
+  int flags;
+  float* y;            // GEMM1: [M_cap, I]
+  uint32_t* rowmax;    // GEMM1: [M_cap]
+  void* rows_out;      // GEMM2: [M_cap, N]
+  int out_dtype;
+  int32_t* acc_dbg;    // [M_cap, N], nullable
+};
+
+// source row of sorted row r of group g
+template <int KIND>
+__device__ __forceinline__ int source_row(const GemmArgs& a, int g, int r) {
+  if constexpr (KIND == 2) {
+    return r;
+  } else {
+    if (g >= a.G) return r - a.offsets[a.G];
+    if (a.sorted_src == nullptr) return r;
+    int s = a.sorted_src[r];
+    return (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? s / a.K : s % a.T;
+  }
+}
+
+// Epilogue of one 16x16 gate/up tile pair of GEMM1.  rows: row0 + rbase + i (i < 4) for this lane.
+__device__ __forceinline__ void epilogue_gemm1(const GemmArgs& a, int g, const float* __restrict__ wsc, int I, int n,
+                                               int row0, int rbase, int nrows, const float* ts, v4i accg, v4i accu,
+                                               float* rmax) {
+  const float wg = wsc[n], wu = wsc[I + n];
+  const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int rr = rbase + i;
+    if (rr < nrows) {
+      float dg = ((float)accg[i] * wg) * ts[i];
+      float du = ((float)accu[i] * wu) * ts[i];
+      if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+      float yv = silu_spec(dg) * du;
+      if (bf) yv = round_bf16(yv);
+      size_t m = (size_t)(row0 + rr);
+      a.y[m * I + n] = yv;
+      rmax[i] = fmaxf(rmax[i], fabsf(yv));
+      if (a.acc_dbg) {
+        a.acc_dbg[m * (size_t)a.N + n] = accg[i];
+        a.acc_dbg[m * (size_t)a.N + I + n] = accu[i];
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float* __restrict__ wsc, int n, int row0,
+                                               int rbase, int nrows, const float* ts, v4i acc) {
+  const float ws = wsc[n];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int rr = rbase + i;
+    if (rr < nrows) {
+      float o = ((float)acc[i] * ws) * ts[i];
+      size_t m = (size_t)(row0 + rr);
+      if (a.out_dtype == OMNI_DT_F32) ((float*)a.rows_out)[m * (size_t)a.N + n] = o;
+      else ((uint16_t*)a.rows_out)[m * (size_t)a.N + n] = f32_to_bf16(o);
+      if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + n] = acc[i];
+    }
+  }
+}
+
+// fold the lane's row maxima over the 16 lanes that hold the same rows, then one atomic per row
+__device__ __forceinline__ void flush_rowmax(const GemmArgs& a, int row0, int rbase, int nrows, float* rmax) {
+  const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float m = row16_allmax_f(rmax[i]);
+    int rr = rbase + i;
+    if ((lane & 15) == 0 && rr < nrows) atomicMax(&a.rowmax[row0 + rr], __float_as_uint(m));
+  }
+}
+
+// =====================================================================================
+// gemm_stream
+//   KIND 1: a wavefront owns NT (gate, up) strip pairs; KIND 2: NT strips.
+//   MT: 16-row tiles per block (block covers up to 16*MT rows of one group).
+//   D : k-steps of B kept in flight per wavefront (multiple of 4).
+// =====================================================================================
+template <int KIND, int MT, int NT, int D>
+__global__ __launch_bounds__(256) void gemm_stream(GemmArgs a) {
+  constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
+  constexpr int BM = 16 * MT;
+  __shared__ v4i lds_a[2][MT * 4 * WAVE];
+
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int w = threadIdx.x / WAVE;
+  RowBlock rb;
+  if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, blockIdx.y, rb)) return;
+  const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
+  const int mt_cnt = (nrows + 15) / 16;
+  const int nk64 = a.Kdim / 64;
+  const int I = (KIND == 1) ? a.N / 2 : 0;
+
+  const int8_t* wbase = (g < a.G) ? a.w + (size_t)g * a.Kdim * a.N : a.w_extra;
+  const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
+
+  // strips of this wavefront
+  int strip[NBF];
+  const int8_t* bp[NBF];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int q = (blockIdx.x * 4 + w) * NT + t;
+    if constexpr (KIND == 1) {
+      strip[2 * t] = q;
+      strip[2 * t + 1] = I / 16 + q;
+    } else {
+      strip[t] = q;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NBF; ++j) bp[j] = wbase + (size_t)strip[j] * nk64 * 1024 + lane * 16;
+
+  // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile
+  const int8_t* arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int rr = mt * 16 + (lane & 15);
+    arow[mt] = nullptr;
+    if (rr < nrows) arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (lane >> 4) * 16;
+  }
+
+  v4i acc[MT][NBF];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < NBF; ++j) acc[mt][j] = (v4i){0, 0, 0, 0};
+
+  // ---- prologue: A chunk 0 -> LDS, first D k-steps of B -> ring
+  v4i areg[MT];
+  {
+    const int ks = w;  // wavefront w stages k-step 4c + w of every chunk c
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      areg[mt] = (v4i){0, 0, 0, 0};
+      if (ks < nk64 && arow[mt]) areg[mt] = *(const v4i*)(arow[mt] + (size_t)ks * 64);
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) lds_a[0][(mt * 4 + w) * WAVE + lane] = areg[mt];
+  }
+  v4i ring[D][NBF];
+#pragma unroll
+  for (int s = 0; s < D; ++s)
+#pragma unroll
+    for (int j = 0; j < NBF; ++j) {
+      ring[s][j] = (v4i){0, 0, 0, 0};
+      if (s < nk64) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
+    }
+  __syncthreads();
+
+  for (int step = 0; step < nk64; step += D) {
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+      const int st = step + s;
+      if (st < nk64) {
+        const int c = st >> 2;
+        const int kk = s & 3;
+        if (kk == 0) {
+          // fetch this wavefront's share of the next A chunk while this one is consumed
+          const int ks = (c + 1) * 4 + w;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            areg[mt] = (v4i){0, 0, 0, 0};
+            if (ks < nk64 && arow[mt]) areg[mt] = *(const v4i*)(arow[mt] + (size_t)ks * 64);
+          }
+        }
+        v4i b[NBF];
+#pragma unroll
+        for (int j = 0; j < NBF; ++j) {
+          b[j] = ring[s][j];
+          if (st + D < nk64) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)(st + D) * 1024));
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          if (mt < mt_cnt) {
+            v4i af = lds_a[c & 1][(mt * 4 + kk) * WAVE + lane];
+#pragma unroll
+            for (int j = 0; j < NBF; ++j) acc[mt][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b[j], acc[mt][j], 0, 0, 0);
+          }
+        }
+        if (kk == 3 && st + 1 < nk64) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) lds_a[(c + 1) & 1][(mt * 4 + w) * WAVE + lane] = areg[mt];
+          __syncthreads();
+        }
+      }
+    }
+  }
+
+  // ---- epilogue
+  const int col = lane & 15;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (mt < mt_cnt) {
+      const int rbase = mt * 16 + 4 * (lane >> 4);
+      float ts[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int rr = rbase + i;
+        ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
+      }
+      if constexpr (KIND == 1) {
+        float rmax[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          epilogue_gemm1(a, g, wsc, I, strip[2 * t] * 16 + col, row0, rbase, nrows, ts, acc[mt][2 * t], acc[mt][2 * t + 1], rmax);
+        flush_rowmax(a, row0, rbase, nrows, rmax);
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsc, strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
+      }
+    }
+  }
+}
+
+// =====================================================================================
+// gemm_tile: block tile 256 rows x 128 channels (GEMM1: 64 gate + 64 up), k-step 64.
+//   four wavefronts as 2 (rows) x 2 (channels); a wavefront holds 8 x 4 accumulator tiles.
+// =====================================================================================
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void gemm_tile(GemmArgs a) {
+  constexpr int BM = 256, MTW = 8, NTW = 4;
+  __shared__ v4i lds_a[2][16 * WAVE];  // 16 fragments of 16 rows x 64 k
+  __shared__ v4i lds_b[2][8 * WAVE];   // 8 strips x 64 k
+
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int w = threadIdx.x / WAVE;
+  const int wm = w >> 1, wn = w & 1;
+  RowBlock rb;
+  if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, blockIdx.y, rb)) return;
+  const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
+  const int nk64 = a.Kdim / 64;
+  const int I = (KIND == 1) ? a.N / 2 : 0;
+
+  const int8_t* wbase = (g < a.G) ? a.w + (size_t)g * a.Kdim * a.N : a.w_extra;
+  const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
+
+  // the block's 8 strips: KIND 1: gate strips 4bx..4bx+3 then up strips; KIND 2: 8bx..8bx+7.
+  // block-level strip j (0..7); wavefront wn uses KIND 1: gate {2wn, 2wn+1}, up {4+2wn, 4+2wn+1};
+  // KIND 2: {4wn .. 4wn+3}.
+  auto strip_of = [&](int j) -> int {
+    if constexpr (KIND == 1) return (j < 4) ? blockIdx.x * 4 + j : I / 16 + blockIdx.x * 4 + (j - 4);
+    else return blockIdx.x * 8 + j;
+  };
+  // staging duties: A fragments 4w..4w+3 (rows 16*(4w+i) + lane%16), B strips 2w, 2w+1
+  const int8_t* arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int rr = (4 * w + i) * 16 + (lane & 15);
+    arow[i] = nullptr;
+    if (rr < nrows) arow[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (lane >> 4) * 16;
+  }
+  const int8_t* bsrc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) bsrc[i] = wbase + (size_t)strip_of(2 * w + i) * nk64 * 1024 + lane * 16;
+
+  int bsel[NTW];  // block-level strip index of each of the wavefront's channel tiles
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) {
+    if constexpr (KIND == 1) bsel[t] = (t < 2) ? 2 * wn + t : 4 + 2 * wn + (t - 2);
+    else bsel[t] = 4 * wn + t;
+  }
+
+  v4i acc[MTW][NTW];
+#pragma unroll
+  for (int mt = 0; mt < MTW; ++mt)
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) acc[mt][t] = (v4i){0, 0, 0, 0};
+
+  v4i areg[4], breg[2];
+  auto fetch = [&](int ks) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      areg[i] = (v4i){0, 0, 0, 0};
+      if (arow[i]) areg[i] = *(const v4i*)(arow[i] + (size_t)ks * 64);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) breg[i] = *(const v4i*)(bsrc[i] + (size_t)ks * 1024);
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_a[buf][(4 * w + i) * WAVE + lane] = areg[i];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) lds_b[buf][(2 * w + i) * WAVE + lane] = breg[i];
+  };
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int mt_lim = min(MTW, (nrows - wm * 128 + 15) / 16);  // row tiles of this wavefront that hold rows
+  for (int ks = 0; ks < nk64; ++ks) {
+    const int buf = ks & 1;
+    if (ks + 1 < nk64) fetch(ks + 1);
+    v4i bf[NTW];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) bf[t] = lds_b[buf][bsel[t] * WAVE + lane];
+#pragma unroll
+    for (int mt = 0; mt < MTW; ++mt) {
+      if (mt < mt_lim) {
+        v4i af = lds_a[buf][(wm * 8 + mt) * WAVE + lane];
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) acc[mt][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf[t], acc[mt][t], 0, 0, 0);
+      }
+    }
+    if (ks + 1 < nk64) {
+      stash(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  const int col = lane & 15;
+#pragma unroll
+  for (int mt = 0; mt < MTW; ++mt) {
+    if (mt < mt_lim) {
+      const int rbase = wm * 128 + mt * 16 + 4 * (lane >> 4);
+      float ts[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int rr = rbase + i;
+        ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
+      }
+      if constexpr (KIND == 1) {
+        float rmax[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          int n = (blockIdx.x * 4 + 2 * wn + t) * 16 + col;
+          epilogue_gemm1(a, g, wsc, I, n, row0, rbase, nrows, ts, acc[mt][t], acc[mt][2 + t], rmax);
+        }
+        flush_rowmax(a, row0, rbase, nrows, rmax);
+      } else {
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) {
+          int n = (blockIdx.x * 8 + 4 * wn + t) * 16 + col;
+          epilogue_gemm2(a, wsc, n, row0, rbase, nrows, ts, acc[mt][t]);
+        }
+      }
+    }
+  }
+}
+
+// =====================================================================================
+// row quantisation of y with the row maximum already known (one wavefront per row)
+// =====================================================================================
+__global__ __launch_bounds__(256) void quant_known_max(const float* __restrict__ y, const uint32_t* __restrict__ rowmax,
+                                                       const int32_t* __restrict__ offsets, int G, int extra_rows, int I,
+                                                       int64_t M_cap, int8_t* __restrict__ hq, float* __restrict__ hs) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t m = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
+  const int64_t total = (int64_t)offsets[G] + extra_rows;
+  if (m >= total || m >= M_cap) return;
+  const float s = __uint_as_float(rowmax[m]) / 127.0f;
+  if (lane == 0) hs[m] = s;
+  const float* yr = y + m * I;
+  int8_t* qr = hq + m * I;
+  for (int c = lane * 4; c < I; c += WAVE * 4) {
+    v4f v = *(const v4f*)(yr + c);
+    uint32_t o = 0;
+    if (s > 0.0f) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o |= ((uint32_t)(quant_i8(v[j], s) & 0xff)) << (8 * j);
+    }
+    *(uint32_t*)(qr + c) = o;
+  }
+}
+
+__global__ __launch_bounds__(256) void zero_u32(uint32_t* p, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// ---------------------------------------------------------------- weight packing
+__global__ __launch_bounds__(256) void pack_weight_kernel(const int8_t* __restrict__ w, int src_layout, int Kdim, int N,
+                                                          int8_t* __restrict__ out) {
+  // one thread per 16-byte fragment piece
+  const int nk64 = Kdim / 64;
+  const size_t per_mat = (size_t)Kdim * N;
+  const size_t piece = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t npieces = per_mat / 16;
+  if (piece >= npieces) return;
+  const int g = blockIdx.y;
+  const int l = (int)(piece % 64);
+  const size_t tile = piece / 64;
+  const int k64 = (int)(tile % nk64);
+  const int n16 = (int)(tile / nk64);
+  const int n = n16 * 16 + (l & 15);
+  const int k0 = k64 * 64 + (l >> 4) * 16;
+  const int8_t* src = w + (size_t)g * per_mat;
+  int8_t v[16];
+  if (src_layout == 1) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = src[(size_t)n * Kdim + k0 + j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = src[(size_t)(k0 + j) * N + n];
+  }
+  int8_t* dst = out + (size_t)g * per_mat + piece * 16;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) dst[j] = v[j];
+}
+
+// ---------------------------------------------------------------- host side dispatch
+struct Plan {
+  bool tile;
+  int mt, nt;  // stream kernel parameters
+};
+
+Plan choose_plan(int kind, int T, int K, int G, int extra_rows, int N_strips_unit) {
+  // expected rows of a busy group
+  int64_t per = (G > 0) ? ((int64_t)T * K + G - 1) / G : 0;
+  if (extra_rows > per) per = extra_rows;
+  if (per > (int64_t)T) per = T;
+  Plan p;
+  p.tile = per > 128;
+  // a block covers 16*mt rows; leave head room over the mean so that a group rarely needs a
+  // second pass over its weights
+  p.mt = per <= 10 ? 1 : (per <= 21 ? 2 : 4);
+  p.nt = 1;
+  (void)kind; (void)N_strips_unit;
+  return p;
+}
+
+template <int KIND, int MT, int NT, int D>
+void launch_stream(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
+  const int BM = 16 * MT;
+  const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
+  int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
+  dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks), block(256);
+  hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
+}
+
+template <int KIND>
+void launch_tile(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
+  const int BM = 256;
+  const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
+  int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
+  const int per_block = (KIND == 1) ? 4 : 8;
+  dim3 grid((unsigned)(units / per_block), (unsigned)mblocks), block(256);
+  hipLaunchKernelGGL((gemm_tile<KIND>), grid, block, 0, st, a);
+}
+
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : dflt;
+}
+
+template <int KIND>
+int dispatch_gemm(const GemmArgs& a, int64_t M_cap, hipStream_t st, const char* what) {
+  // units: KIND 1 -> (gate, up) strip pairs = I/16; KIND 2 -> strips = N/16
+  const int units = (KIND == 1) ? a.N / 32 : a.N / 16;
+  Plan p = choose_plan(KIND, a.T, a.K, a.G, a.extra_rows, units);
+  int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // 1 stream, 2 tile (tuning aid)
+  if (force == 1) p.tile = false;
+  if (force == 2) p.tile = true;
+  const int tile_units = (KIND == 1) ? 4 : 8;
+  if (p.tile && units % tile_units != 0) p.tile = false;
+  if (p.tile) {
+    launch_tile<KIND>(a, M_cap, units, st);
+  } else {
+    if (units % 4 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: output channels %d not a multiple of %d", what, a.N, KIND == 1 ? 128 : 64);
+    int mt = env_int("OMNI_MOE_STREAM_MT", p.mt);
+    if constexpr (KIND == 1) {
+      if (mt <= 1) launch_stream<1, 1, 1, 8>(a, M_cap, units, st);
+      else if (mt == 2) launch_stream<1, 2, 1, 8>(a, M_cap, units, st);
+      else launch_stream<1, 4, 1, 4>(a, M_cap, units, st);
+    } else {
+      const bool nt4 = units % 16 == 0, nt2 = units % 8 == 0;
+      if (nt4) {
+        if (mt <= 1) launch_stream<2, 1, 4, 4>(a, M_cap, units, st);
+        else if (mt == 2) launch_stream<2, 2, 4, 4>(a, M_cap, units, st);
+        else launch_stream<2, 4, 4, 4>(a, M_cap, units, st);
+      } else if (nt2) {
+        if (mt <= 2) launch_stream<2, 2, 2, 4>(a, M_cap, units, st);
+        else launch_stream<2, 4, 2, 4>(a, M_cap, units, st);
+      } else {
+        if (mt <= 2) launch_stream<2, 2, 1, 4>(a, M_cap, units, st);
+        else launch_stream<2, 4, 1, 4>(a, M_cap, units, st);
+      }
+    }
+  }
+  OMNI_CHECK_LAUNCH(what);
+  return OMNI_OK;
+}
+
+int check_group_args(const char* what, const int32_t* offsets, int G, int H, int I, int64_t M_cap, int extra_rows,
+                     const void* w_extra, const void* w_extra_scale) {
+  if (G < 0 || H <= 0 || I <= 0 || M_cap < 0 || extra_rows < 0) OMNI_FAIL(OMNI_E_INVALID, "%s: bad sizes G=%d H=%d I=%d M_cap=%lld", what, G, H, I, (long long)M_cap);
+  if (!offsets) OMNI_FAIL(OMNI_E_INVALID, "%s: offsets is null", what);
+  if (H % 64 != 0 || I % 64 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: H=%d and I=%d must be multiples of 64", what, H, I);
+  if (extra_rows > 0 && (!w_extra || !w_extra_scale)) OMNI_FAIL(OMNI_E_INVALID, "%s: extra group without weights", what);
+  if (M_cap > 0x7fffffffLL) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: M_cap too large", what);
+  return OMNI_OK;
+}
+
+}  // namespace
+
+extern "C" size_t omni_moe_gemm1_workspace_bytes(int64_t M_cap, int I) {
+  if (M_cap < 0 || I <= 0) return 0;
+  size_t y = (size_t)M_cap * I * sizeof(float);
+  size_t rm = (((size_t)M_cap * sizeof(uint32_t)) + 255) / 256 * 256;
+  return y + rm + 256;
+}
+
+extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src,
+                                           int idx_mode, int T, int K, const int8_t* w13_packed,
+                                           const float* w13_scale, const int8_t* w13_extra,
+                                           const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G,
+                                           int H, int I, int64_t M_cap, int flags, int8_t* h_q, float* h_scale,
+                                           int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream) {
+  int rc = check_group_args("gemm1", offsets, G, H, I, M_cap, extra_rows, w13_extra, w13_extra_scale);
+  if (rc) return rc;
+  if (M_cap == 0) return OMNI_OK;
+  if (!x_q || !x_scale || !h_q || !h_scale || (G > 0 && (!w13_packed || !w13_scale))) OMNI_FAIL(OMNI_E_INVALID, "gemm1: null pointer");
+  if (T <= 0 || K <= 0) OMNI_FAIL(OMNI_E_INVALID, "gemm1: bad T=%d K=%d", T, K);
+  if (ws_bytes < omni_moe_gemm1_workspace_bytes(M_cap, I) || !workspace) OMNI_FAIL(OMNI_E_WORKSPACE, "gemm1: workspace %zu < %zu", ws_bytes, omni_moe_gemm1_workspace_bytes(M_cap, I));
+  if (((uintptr_t)x_q % 16) || ((uintptr_t)w13_packed % 16) || ((uintptr_t)w13_extra % 16) || ((uintptr_t)workspace % 16) || ((uintptr_t)h_q % 4))
+    OMNI_FAIL(OMNI_E_INVALID, "gemm1: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  float* y = (float*)workspace;
+  uint32_t* rowmax = (uint32_t*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
+  hipLaunchKernelGGL(zero_u32, dim3((unsigned)((M_cap + 255) / 256)), dim3(256), 0, st, rowmax, M_cap);
+  GemmArgs a{};
+  a.a_q = x_q; a.a_scale = x_scale; a.sorted_src = sorted_src; a.idx_mode = idx_mode; a.T = T; a.K = K;
+  a.w = w13_packed; a.w_scale = w13_scale; a.w_extra = w13_extra; a.w_extra_scale = w13_extra_scale;
+  a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = H; a.N = 2 * I; a.flags = flags;
+  a.y = y; a.rowmax = rowmax; a.acc_dbg = acc_dbg;
+  rc = dispatch_gemm<1>(a, M_cap, st, "gemm1");
+  if (rc) return rc;
+  hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax, offsets, G,
+                     extra_rows, I, M_cap, h_q, h_scale);
+  OMNI_CHECK_LAUNCH("gemm1 quant");
+  return OMNI_OK;
+}
+
+extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed,
+                                      const float* w2_scale, const int8_t* w2_extra, const float* w2_extra_scale,
+                                      int extra_rows, const int32_t* offsets, int G, int H, int I, int64_t M_cap,
+                                      int out_dtype, void* rows_out, int32_t* acc_dbg, void* stream) {
+  int rc = check_group_args("gemm2", offsets, G, H, I, M_cap, extra_rows, w2_extra, w2_extra_scale);
+  if (rc) return rc;
+  if (M_cap == 0) return OMNI_OK;
+  if (!h_q || !h_scale || !rows_out || (G > 0 && (!w2_packed || !w2_scale))) OMNI_FAIL(OMNI_E_INVALID, "gemm2: null pointer");
+  if (out_dtype != OMNI_DT_BF16 && out_dtype != OMNI_DT_F32) OMNI_FAIL(OMNI_E_INVALID, "gemm2: out_dtype %d", out_dtype);
+  if (((uintptr_t)h_q % 16) || ((uintptr_t)w2_packed % 16) || ((uintptr_t)w2_extra % 16)) OMNI_FAIL(OMNI_E_INVALID, "gemm2: pointers must be 16-byte aligned");
+  GemmArgs a{};
+  a.a_q = h_q; a.a_scale = h_scale; a.sorted_src = nullptr; a.idx_mode = 0;
+  // T and K only steer the kernel choice here: rows per group ~ M_cap / groups
+  a.T = (int)M_cap; a.K = 1;
+  a.w = w2_packed; a.w_scale = w2_scale; a.w_extra = w2_extra; a.w_extra_scale = w2_extra_scale;
+  a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = I; a.N = H; a.flags = 0;
+  a.rows_out = rows_out; a.out_dtype = out_dtype; a.acc_dbg = acc_dbg;
+  return dispatch_gemm<2>(a, M_cap, (hipStream_t)stream, "gemm2");
+}
+
+extern "C" int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N, int8_t* packed,
+                                    void* stream) {
+  if (G <= 0 || Kdim <= 0 || N <= 0) OMNI_FAIL(OMNI_E_INVALID, "pack_weight: bad sizes");
+  if (!w || !packed) OMNI_FAIL(OMNI_E_INVALID, "pack_weight: null pointer");
+  if (Kdim % 64 != 0 || N % 16 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "pack_weight: Kdim=%d must be a multiple of 64 and N=%d of 16", Kdim, N);
+  if (src_layout != 0 && src_layout != 1) OMNI_FAIL(OMNI_E_INVALID, "pack_weight: src_layout %d", src_layout);
+  size_t npieces = (size_t)Kdim * N / 16;
+  dim3 grid((unsigned)((npieces + 255) / 256), (unsigned)G), block(256);
+  hipLaunchKernelGGL(pack_weight_kernel, grid, block, 0, (hipStream_t)stream, w, src_layout, Kdim, N, packed);
+  OMNI_CHECK_LAUNCH("pack_weight");
+  return OMNI_OK;
+}

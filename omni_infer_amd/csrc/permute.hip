@@ -1,0 +1,258 @@
+// Stable counting sort of the (token, k) assignments by local expert id.
+//
+// Assignments are numbered p = n*K + k.  Bucket e < G is local expert lo + e, bucket G collects
+// the assignments whose expert is outside [lo, hi) ("dropped"); the dropped bucket sorts last.
+// A block of four wavefronts ranks a chunk of assignments: each wavefront walks its part of the
+// chunk 64 assignments at a time, finds the lanes that hold the same bucket with one ballot per
+// bucket-id bit, and keeps a running per-bucket count in an LDS histogram (one per wavefront).
+// An exclusive prefix over wavefronts, blocks and buckets then gives every assignment its slot.
+// Small inputs (<= 4096 assignments) are sorted by one block in one launch; larger ones take a
+// count launch, a one-block scan launch and a scatter launch.
+#include "common.h"
+
+namespace {
+
+constexpr int GMAX = 256;        // local experts per call
+constexpr int NB = GMAX + 1;     // buckets incl. the dropped one
+constexpr int CH_MULTI = 1024;   // assignments per block in the multi-block path
+constexpr int CH_SINGLE = 4096;  // largest input of the single-block path
+
+struct PermArgs {
+  const int32_t* ids;
+  int n, T, K, lo, G, idx_mode;
+  int32_t* sorted_src;
+  int32_t* src_to_dst;
+  int32_t* counts;
+  int32_t* offsets;
+  int32_t* blk_hist;  // [nblk][NB] counts, then (after the scan) exclusive block bases
+  int nblk;
+};
+
+__device__ __forceinline__ int bucket_of(int id, int lo, int G) {
+  int e = id - lo;
+  return (e >= 0 && e < G) ? e : G;
+}
+
+// Ranks the chunk [base, base+len): lrank[i] = number of earlier assignments of the same bucket
+// inside the same wavefront's part; whist[w][b] = count of bucket b in wavefront w's part.
+__device__ __forceinline__ void rank_chunk(const PermArgs& a, int base, int len, int passes, int (*whist)[NB],
+                                           int* lrank) {
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+  for (int i = threadIdx.x; i < 4 * NB; i += 256) (&whist[0][0])[i] = 0;
+  __syncthreads();
+  const int nbits = 32 - __clz(a.G);
+  const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int j = 0; j < passes; ++j) {
+    int i = (w * passes + j) * WAVE + lane;
+    bool valid = i < len;
+    int b = valid ? bucket_of(a.ids[base + i], a.lo, a.G) : 0;
+    uint64_t peers = __ballot(valid);
+    for (int bit = 0; bit < nbits; ++bit) {
+      uint64_t m = __ballot((b >> bit) & 1);
+      peers &= ((b >> bit) & 1) ? m : ~m;
+    }
+    if (valid) {
+      // lanes of one wavefront run these two LDS accesses in program order: every peer reads
+      // the running count before the first peer replaces it
+      volatile int* cnt = &whist[w][b];
+      int r = __popcll(peers & lt);
+      int start = *cnt;
+      lrank[i] = start + r;
+      if (r == 0) *cnt = start + __popcll(peers);
+    }
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ int src_index(const PermArgs& a, int p) {
+  if (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) return p;
+  int n = p / a.K, k = p - n * a.K;
+  return k * a.T + n;
+}
+
+// Scatter of the chunk, given for every bucket the slot of the chunk's first assignment of it.
+__device__ __forceinline__ void scatter_chunk(const PermArgs& a, int base, int len, int passes, int (*whist)[NB],
+                                              const int* lrank, const int* bucket_slot0) {
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+  for (int j = 0; j < passes; ++j) {
+    int i = (w * passes + j) * WAVE + lane;
+    if (i < len) {
+      int b = bucket_of(a.ids[base + i], a.lo, a.G);
+      int slot = bucket_slot0[b] + lrank[i];
+      for (int ww = 0; ww < w; ++ww) slot += whist[ww][b];
+      int src = src_index(a, base + i);
+      a.sorted_src[slot] = src;
+      a.src_to_dst[src] = (b < a.G) ? slot : -1;
+    }
+  }
+}
+
+// exclusive scan of tot[0..nb) by wavefront 0 into off[0..nb]; off[nb] = grand total
+__device__ __forceinline__ void wave0_excl_scan(const int* tot, int* off, int nb) {
+  if (threadIdx.x < WAVE) {
+    const int lane = threadIdx.x;
+    const int per = (nb + WAVE - 1) / WAVE;
+    int mine = 0;
+    for (int j = 0; j < per; ++j) {
+      int b = lane * per + j;
+      if (b < nb) mine += tot[b];
+    }
+    int incl = wave_incl_scan_i(mine, lane);
+    int run = incl - mine;
+    for (int j = 0; j < per; ++j) {
+      int b = lane * per + j;
+      if (b < nb) {
+        off[b] = run;
+        run += tot[b];
+      }
+    }
+    if (lane == WAVE - 1) off[nb] = incl;
+  }
+}
+
+__global__ __launch_bounds__(256) void permute_single(PermArgs a) {
+  __shared__ int whist[4][NB];
+  __shared__ int lrank[CH_SINGLE];
+  __shared__ int tot[NB];
+  __shared__ int off[NB + 1];
+  const int passes = (a.n + 255) / 256;
+  rank_chunk(a, 0, a.n, passes, whist, lrank);
+  const int nb = a.G + 1;
+  for (int b = threadIdx.x; b < nb; b += 256) tot[b] = whist[0][b] + whist[1][b] + whist[2][b] + whist[3][b];
+  __syncthreads();
+  wave0_excl_scan(tot, off, nb);
+  __syncthreads();
+  for (int b = threadIdx.x; b < a.G; b += 256) {
+    a.counts[b] = tot[b];
+    a.offsets[b] = off[b];
+  }
+  if (threadIdx.x == 0) a.offsets[a.G] = off[a.G];
+  scatter_chunk(a, 0, a.n, passes, whist, lrank, off);
+}
+
+__global__ __launch_bounds__(256) void permute_count(PermArgs a) {
+  __shared__ int whist[4][NB];
+  __shared__ int lrank[CH_MULTI];
+  const int base = blockIdx.x * CH_MULTI;
+  const int len = min(CH_MULTI, a.n - base);
+  rank_chunk(a, base, len, CH_MULTI / 256, whist, lrank);
+  for (int b = threadIdx.x; b <= a.G; b += 256)
+    a.blk_hist[(size_t)blockIdx.x * NB + b] = whist[0][b] + whist[1][b] + whist[2][b] + whist[3][b];
+}
+
+// one block: per bucket exclusive prefix over blocks (in place), then the prefix over buckets
+__global__ __launch_bounds__(256) void permute_scan(PermArgs a) {
+  __shared__ int tot[NB];
+  __shared__ int off[NB + 1];
+  const int nb = a.G + 1;
+  for (int b = threadIdx.x; b < nb; b += 256) {
+    int run = 0;
+    for (int k = 0; k < a.nblk; ++k) {
+      int c = a.blk_hist[(size_t)k * NB + b];
+      a.blk_hist[(size_t)k * NB + b] = run;
+      run += c;
+    }
+    tot[b] = run;
+  }
+  __syncthreads();
+  wave0_excl_scan(tot, off, nb);
+  __syncthreads();
+  for (int b = threadIdx.x; b < a.G; b += 256) {
+    a.counts[b] = tot[b];
+    a.offsets[b] = off[b];
+  }
+  if (threadIdx.x == 0) a.offsets[a.G] = off[a.G];
+  // bucket bases for the scatter launch live after the block table
+  for (int b = threadIdx.x; b < nb; b += 256) a.blk_hist[(size_t)a.nblk * NB + b] = off[b];
+}
+
+__global__ __launch_bounds__(256) void permute_scatter(PermArgs a) {
+  __shared__ int whist[4][NB];
+  __shared__ int lrank[CH_MULTI];
+  __shared__ int slot0[NB];
+  const int base = blockIdx.x * CH_MULTI;
+  const int len = min(CH_MULTI, a.n - base);
+  rank_chunk(a, base, len, CH_MULTI / 256, whist, lrank);
+  for (int b = threadIdx.x; b <= a.G; b += 256)
+    slot0[b] = a.blk_hist[(size_t)a.nblk * NB + b] + a.blk_hist[(size_t)blockIdx.x * NB + b];
+  __syncthreads();
+  scatter_chunk(a, base, len, CH_MULTI / 256, whist, lrank, slot0);
+}
+
+struct GatherArgs {
+  const uint8_t* x;
+  int64_t row_bytes;
+  const float* x_scale;
+  const int32_t* sorted_src;
+  const int32_t* offsets;
+  int n_local, T, K, idx_mode;
+  uint8_t* rows_out;
+  float* scale_out;
+};
+
+// one block per sorted slot; slots past the kept total copy nothing
+__global__ __launch_bounds__(256) void gather_rows_kernel(GatherArgs g) {
+  const int m = blockIdx.x;
+  if (m >= g.offsets[g.n_local]) return;
+  const int src = g.sorted_src[m];
+  const int tok = (g.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? src / g.K : src % g.T;
+  const uint8_t* s = g.x + (size_t)tok * g.row_bytes;
+  uint8_t* d = g.rows_out + (size_t)m * g.row_bytes;
+  if ((g.row_bytes % 16 == 0) && ((uintptr_t)g.x % 16 == 0) && ((uintptr_t)g.rows_out % 16 == 0)) {
+    for (int64_t i = threadIdx.x; i < g.row_bytes / 16; i += 256) ((v4i*)d)[i] = ((const v4i*)s)[i];
+  } else {
+    for (int64_t i = threadIdx.x; i < g.row_bytes; i += 256) d[i] = s[i];
+  }
+  if (threadIdx.x == 0 && g.x_scale && g.scale_out) g.scale_out[m] = g.x_scale[tok];
+}
+
+}  // namespace
+
+extern "C" size_t omni_moe_permute_workspace_bytes(int T, int K, int n_local) {
+  (void)n_local;
+  int64_t n = (int64_t)T * K;
+  if (n <= CH_SINGLE) return 256;
+  int64_t nblk = (n + CH_MULTI - 1) / CH_MULTI;
+  return (size_t)((nblk + 1) * NB * sizeof(int32_t));
+}
+
+extern "C" int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode,
+                                int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts, int32_t* offsets,
+                                void* workspace, size_t ws_bytes, void* stream) {
+  if (T < 0 || K <= 0 || hi <= lo) OMNI_FAIL(OMNI_E_INVALID, "permute: bad sizes T=%d K=%d range=[%d,%d)", T, K, lo, hi);
+  const int G = hi - lo;
+  if (G > GMAX) OMNI_FAIL(OMNI_E_UNSUPPORTED, "permute: %d local experts > %d", G, GMAX);
+  if ((int64_t)T * K > 0x7fffffffLL) OMNI_FAIL(OMNI_E_UNSUPPORTED, "permute: T*K overflows int32");
+  if (!counts || !offsets) OMNI_FAIL(OMNI_E_INVALID, "permute: null pointer");
+  if (idx_mode != OMNI_IDX_TOKEN_MAJOR && idx_mode != OMNI_IDX_K_MAJOR) OMNI_FAIL(OMNI_E_INVALID, "permute: bad idx_mode %d", idx_mode);
+  if (T > 0 && (!topk_ids || !sorted_src || !src_to_dst)) OMNI_FAIL(OMNI_E_INVALID, "permute: null pointer");
+  const int n = T * K;
+  if (ws_bytes < omni_moe_permute_workspace_bytes(T, K, G)) OMNI_FAIL(OMNI_E_WORKSPACE, "permute: workspace %zu < %zu", ws_bytes, omni_moe_permute_workspace_bytes(T, K, G));
+  hipStream_t st = (hipStream_t)stream;
+  PermArgs a{topk_ids, n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, (int32_t*)workspace, 0};
+  if (n <= CH_SINGLE) {
+    hipLaunchKernelGGL(permute_single, dim3(1), dim3(256), 0, st, a);
+    OMNI_CHECK_LAUNCH("permute_single");
+    return OMNI_OK;
+  }
+  if (!workspace) OMNI_FAIL(OMNI_E_WORKSPACE, "permute: workspace is null");
+  a.nblk = (n + CH_MULTI - 1) / CH_MULTI;
+  hipLaunchKernelGGL(permute_count, dim3(a.nblk), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(permute_scan, dim3(1), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(permute_scatter, dim3(a.nblk), dim3(256), 0, st, a);
+  OMNI_CHECK_LAUNCH("permute");
+  return OMNI_OK;
+}
+
+extern "C" int omni_moe_gather_rows(const void* x, int elem_bytes, int H, const float* x_scale,
+                                    const int32_t* sorted_src, const int32_t* offsets, int n_local, int T, int K,
+                                    int idx_mode, void* rows_out, float* scale_out, void* stream) {
+  if (T < 0 || K <= 0 || H <= 0 || elem_bytes <= 0 || n_local <= 0) OMNI_FAIL(OMNI_E_INVALID, "gather_rows: bad sizes");
+  if (T == 0) return OMNI_OK;
+  if (!x || !sorted_src || !offsets || !rows_out) OMNI_FAIL(OMNI_E_INVALID, "gather_rows: null pointer");
+  GatherArgs g{(const uint8_t*)x, (int64_t)H * elem_bytes, x_scale, sorted_src, offsets, n_local, T, K, idx_mode,
+               (uint8_t*)rows_out, scale_out};
+  hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((int64_t)T * K)), dim3(256), 0, (hipStream_t)stream, g);
+  OMNI_CHECK_LAUNCH("gather_rows");
+  return OMNI_OK;
+}

@@ -1,0 +1,296 @@
+"""Operator boundary: torch-tensor wrappers over the C ABI of libomni_moe_hip.so.
+
+Each function stands where the reference calls a ``torch_npu.npu_*`` operator on the MoE
+path and keeps that operator's argument meaning; the arithmetic is done by the gfx950 HIP
+kernels.  torch is used for device memory and the current stream only.  Nothing here has a
+CPU or eager fallback: tensors must live on the GPU and the library must be built.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib as L
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("omni_infer_amd operators run on the GPU only (got a CPU tensor)")
+
+
+_DT = {torch.bfloat16: L.OMNI_DT_BF16, torch.float32: L.OMNI_DT_F32, torch.float16: L.OMNI_DT_F16}
+
+
+# ----------------------------------------------------------------------------- routing
+def moe_route(logits: torch.Tensor, bias: Optional[torch.Tensor], top_k: int, n_group: int, topk_group: int,
+              score_fn: str, group_mode: int, masked_fill_zero: bool, weight_from_c: bool, renorm: bool,
+              scale: float, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    _need_gpu(logits, bias)
+    if logits.dim() != 2:
+        raise ValueError("router logits must be [T, E]")
+    logits = logits.float().contiguous()
+    T, E = logits.shape
+    if bias is not None:
+        bias = bias.float().contiguous()
+        if bias.numel() != E:
+            raise ValueError("bias must have one entry per expert")
+    w = torch.empty(T, top_k, dtype=torch.float32, device=logits.device)
+    ids = torch.empty(T, top_k, dtype=torch.int32, device=logits.device)
+    fn = {"softmax": L.OMNI_SCORE_SOFTMAX, "sigmoid": L.OMNI_SCORE_SIGMOID}.get(score_fn)
+    if fn is None:
+        raise ValueError(f"Unsupported scoring function: {score_fn}")
+    rc = L.lib().omni_moe_route(_ptr(logits), _ptr(bias), T, E, int(n_group), int(topk_group), int(top_k), fn,
+                                int(group_mode), int(masked_fill_zero), int(weight_from_c), int(renorm),
+                                float(scale), float(eps), _ptr(w), _ptr(ids), _stream())
+    L.check(rc, "omni_moe_route")
+    return w, ids
+
+
+def _row_idx(T: int, K: int, device) -> torch.Tensor:
+    # row_idx[n, k] = k*T + n (fused_moe.py:80-81, layer.py:352-353)
+    return torch.arange(T * K, device=device, dtype=torch.int32).view(K, T).transpose(0, 1)
+
+
+def npu_moe_gating_top_k(x: torch.Tensor, k: int, bias: Optional[torch.Tensor], k_group: int, group_count: int,
+                         group_select_mode: int = 1, renorm: int = 0, norm_type: int = 1,
+                         routed_scaling_factor: float = 1.0, eps: float = 1e-20):
+    """Stands in for ``torch_npu.npu_moe_gating_top_k`` as called at
+    omni/models/common/layers/moe/fused_moe/layer.py:341-351."""
+    if renorm != 0:
+        raise ValueError("npu_moe_gating_top_k: only renorm=0 (score, then top-k) is supported")
+    w, ids = moe_route(x, bias, k, group_count, k_group, "sigmoid" if norm_type == 1 else "softmax",
+                       L.OMNI_GROUP_TOP2SUM if group_select_mode == 1 else L.OMNI_GROUP_MAX,
+                       masked_fill_zero=False, weight_from_c=False, renorm=True,
+                       scale=routed_scaling_factor, eps=eps)
+    return w, ids, None
+
+
+def npu_moe_gating_top_k_softmax(x: torch.Tensor, k: int):
+    """Stands in for ``torch_npu.npu_moe_gating_top_k_softmax`` (fused_moe.py:29)."""
+    w, ids = moe_route(x, None, k, 1, 1, "softmax", L.OMNI_GROUP_MAX, False, False, False, 1.0, 0.0)
+    return w, ids, _row_idx(x.shape[0], k, x.device)
+
+
+# ----------------------------------------------------------------------------- quant
+def npu_dynamic_quant(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Stands in for ``torch_npu.npu_dynamic_quant`` (deepseek_moe.py:247,323;
+    compressed_tensors_moe.py:241,247; schemes/compressed_tensors_w8a8_int8.py:97)."""
+    _need_gpu(x)
+    if x.dtype not in _DT:
+        raise ValueError(f"npu_dynamic_quant: unsupported dtype {x.dtype}")
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1])
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    rows, cols = x2.shape
+    q = torch.empty(rows, cols, dtype=torch.int8, device=x.device)
+    s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    rc = L.lib().omni_dynamic_quant(_ptr(x2), _DT[x.dtype], rows, cols, x2.stride(0) if rows > 1 else cols,
+                                    _ptr(q), _ptr(s), _stream())
+    L.check(rc, "omni_dynamic_quant")
+    return q.view(shape), s.view(shape[:-1])
+
+
+# ----------------------------------------------------------------------------- permutation
+class Permutation:
+    """Result of sorting the (token, k) assignments by local expert."""
+    __slots__ = ("sorted_src", "src_to_dst", "counts", "offsets", "T", "K", "n_local", "idx_mode")
+
+
+def moe_permute(topk_ids: torch.Tensor, lo: int, hi: int, idx_mode: int = L.OMNI_IDX_TOKEN_MAJOR) -> Permutation:
+    _need_gpu(topk_ids)
+    if topk_ids.dtype != torch.int32:
+        topk_ids = topk_ids.to(torch.int32)
+    topk_ids = topk_ids.contiguous()
+    T, K = topk_ids.shape
+    G = hi - lo
+    dev = topk_ids.device
+    p = Permutation()
+    p.T, p.K, p.n_local, p.idx_mode = T, K, G, idx_mode
+    p.sorted_src = torch.empty(max(T * K, 1), dtype=torch.int32, device=dev)
+    p.src_to_dst = torch.empty(max(T * K, 1), dtype=torch.int32, device=dev)
+    p.counts = torch.empty(G, dtype=torch.int32, device=dev)
+    p.offsets = torch.empty(G + 1, dtype=torch.int32, device=dev)
+    ws_bytes = L.lib().omni_moe_permute_workspace_bytes(T, K, G)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    rc = L.lib().omni_moe_permute(_ptr(topk_ids), T, K, lo, hi, idx_mode, _ptr(p.sorted_src), _ptr(p.src_to_dst),
+                                  _ptr(p.counts), _ptr(p.offsets), _ptr(ws), ws_bytes, _stream())
+    L.check(rc, "omni_moe_permute")
+    return p
+
+
+def moe_gather_rows(x: torch.Tensor, x_scale: Optional[torch.Tensor], p: Permutation):
+    _need_gpu(x)
+    x = x.contiguous()
+    T, H = x.shape
+    rows = torch.zeros(T * p.K, H, dtype=x.dtype, device=x.device)
+    sc = torch.zeros(T * p.K, dtype=torch.float32, device=x.device) if x_scale is not None else None
+    rc = L.lib().omni_moe_gather_rows(_ptr(x), x.element_size(), H, _ptr(x_scale), _ptr(p.sorted_src),
+                                      _ptr(p.offsets), p.n_local, T, p.K, p.idx_mode, _ptr(rows), _ptr(sc), _stream())
+    L.check(rc, "omni_moe_gather_rows")
+    return rows, sc
+
+
+def npu_moe_init_routing_v2(x: torch.Tensor, expert_idx: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                            active_expert_range=None, expert_num: int = 0, **_unused):
+    """Stands in for ``torch_npu.npu_moe_init_routing_v2`` with ``row_idx_type=1``,
+    ``expert_tokens_num_type=1``, ``quant_mode=-1`` (fused_moe.py:514-515): returns
+    (sorted rows, expanded_x_idx, per-expert counts int64, gathered scale)."""
+    lo, hi = active_expert_range if active_expert_range is not None else (0, expert_num)
+    p = moe_permute(expert_idx, lo, hi, L.OMNI_IDX_TOKEN_MAJOR)
+    rows, sc = moe_gather_rows(x, scale, p)
+    return rows, p.sorted_src, p.counts.to(torch.int64), sc
+
+
+def npu_moe_init_routing(x: torch.Tensor, row_idx: torch.Tensor, expert_idx: torch.Tensor, active_num: int,
+                         num_experts: int = 256):
+    """Stands in for ``torch_npu.npu_moe_init_routing`` (compressed_tensors_moe.py:235-236):
+    returns (sorted rows, expanded_src_to_dst_row indexed by k*T+n, sorted expert ids).
+    ``row_idx`` must be the reference's k*T+n numbering (the only one it ever builds,
+    compressed_tensors_moe.py:186-187); ``num_experts`` bounds the expert ids (no host sync)."""
+    T, K = expert_idx.shape
+    p = moe_permute(expert_idx, 0, num_experts, L.OMNI_IDX_K_MAJOR)
+    rows, _ = moe_gather_rows(x, None, p)
+    sorted_ids = torch.repeat_interleave(torch.arange(p.n_local, device=x.device, dtype=torch.int32),
+                                         p.counts.to(torch.int64), output_size=T * K)
+    return rows, p.src_to_dst, sorted_ids
+
+
+def npu_moe_compute_expert_tokens(sorted_expert_idx: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """Stands in for ``torch_npu.npu_moe_compute_expert_tokens`` (compressed_tensors_moe.py:237):
+    cumulative number of rows up to and including each expert."""
+    return torch.cumsum(torch.bincount(sorted_expert_idx.to(torch.int64), minlength=num_experts), 0).to(torch.int32)
+
+
+_DENSE_OFFSETS = {}
+
+
+def dense_offsets(M: int, device) -> torch.Tensor:
+    """[0, M] int32 on the device: the row grouping of a dense (one group) GEMM.  Cached so that
+    the steady state issues no host-to-device copy."""
+    key = (int(M), str(device))
+    t = _DENSE_OFFSETS.get(key)
+    if t is None:
+        t = torch.tensor([0, int(M)], dtype=torch.int32, device=device)
+        _DENSE_OFFSETS[key] = t
+    return t
+
+
+# ----------------------------------------------------------------------------- weights
+def pack_weight(w: torch.Tensor, src_layout: int) -> torch.Tensor:
+    """One-off re-layout of int8 weights into the frag16 format the GEMM kernels stream
+    (the analogue of ``npu_format_cast(w, 29)``, compressed_tensors_moe.py:97-99).
+    src_layout 0: w is [G, Kdim, N]; 1: w is [G, N, Kdim]."""
+    _need_gpu(w)
+    if w.dtype != torch.int8:
+        raise ValueError("pack_weight expects int8 weights")
+    if w.dim() == 2:
+        w = w.unsqueeze(0)
+    w = w.contiguous()
+    G = w.shape[0]
+    Kdim, N = (w.shape[1], w.shape[2]) if src_layout == 0 else (w.shape[2], w.shape[1])
+    out = torch.empty(G, Kdim * N, dtype=torch.int8, device=w.device)
+    rc = L.lib().omni_moe_pack_weight(_ptr(w), src_layout, G, Kdim, N, _ptr(out), _stream())
+    L.check(rc, "omni_moe_pack_weight")
+    return out
+
+
+# ----------------------------------------------------------------------------- GEMMs
+def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_src: Optional[torch.Tensor],
+                               idx_mode: int, K: int, w13_packed: torch.Tensor, w13_scale: torch.Tensor,
+                               offsets: torch.Tensor, H: int, I: int, M_cap: int,
+                               extra: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, extra_rows: int = 0,
+                               bf16_intermediate: bool = False, want_acc: bool = False):
+    """GEMM1 + dequant + SwiGLU + requant: ``npu_grouped_matmul(int32)`` +
+    ``npu_dequant_swiglu_quant`` (fused_moe.py:531-534, :670-677).  Returns (h_q, h_scale, acc)."""
+    _need_gpu(x_q, x_scale, w13_packed, w13_scale, offsets)
+    dev = x_q.device
+    T = x_q.shape[0]
+    G = offsets.numel() - 1
+    h_q = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
+    h_s = torch.empty(M_cap, dtype=torch.float32, device=dev)
+    acc = torch.zeros(M_cap, 2 * I, dtype=torch.int32, device=dev) if want_acc else None
+    ws_bytes = L.lib().omni_moe_gemm1_workspace_bytes(M_cap, I)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ew, es = extra if extra is not None else (None, None)
+    rc = L.lib().omni_moe_gemm1_swiglu_quant(
+        _ptr(x_q), _ptr(x_scale), _ptr(sorted_src), idx_mode, T, K, _ptr(w13_packed), _ptr(w13_scale), _ptr(ew),
+        _ptr(es), extra_rows, _ptr(offsets), G, H, I, M_cap, L.OMNI_GEMM1_BF16_INTERMEDIATE if bf16_intermediate else 0,
+        _ptr(h_q), _ptr(h_s), _ptr(acc), _ptr(ws), ws_bytes, _stream())
+    L.check(rc, "omni_moe_gemm1_swiglu_quant")
+    return h_q, h_s, acc
+
+
+def grouped_gemm2_dequant(h_q: torch.Tensor, h_scale: torch.Tensor, w2_packed: torch.Tensor, w2_scale: torch.Tensor,
+                          offsets: torch.Tensor, H: int, I: int, out_dtype: torch.dtype = torch.bfloat16,
+                          extra: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, extra_rows: int = 0,
+                          want_acc: bool = False):
+    """GEMM2 + dequant: ``npu_grouped_matmul(scale=, per_token_scale=, output_dtype=bf16)``
+    (fused_moe.py:570-574, :681-685).  Returns (rows [M_cap, H], acc)."""
+    _need_gpu(h_q, h_scale, w2_packed, w2_scale, offsets)
+    dev = h_q.device
+    M_cap = h_q.shape[0]
+    G = offsets.numel() - 1
+    rows = torch.zeros(M_cap, H, dtype=out_dtype, device=dev)
+    acc = torch.zeros(M_cap, H, dtype=torch.int32, device=dev) if want_acc else None
+    ew, es = extra if extra is not None else (None, None)
+    rc = L.lib().omni_moe_gemm2_dequant(_ptr(h_q), _ptr(h_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(ew), _ptr(es),
+                                        extra_rows, _ptr(offsets), G, H, I, M_cap, _DT[out_dtype], _ptr(rows),
+                                        _ptr(acc), _stream())
+    L.check(rc, "omni_moe_gemm2_dequant")
+    return rows, acc
+
+
+def moe_combine(rows: torch.Tensor, topk_w: torch.Tensor, src_to_dst: torch.Tensor, idx_mode: int, order: int,
+                init: Optional[torch.Tensor] = None, post_add: Optional[torch.Tensor] = None,
+                post_add_row0: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Weighted un-permute: ``npu_moe_finalize_routing`` (compressed_tensors_moe.py:253;
+    deepseek_moe.py:292-301) and the routing half of ``npu_grouped_matmul_finalize_routing``
+    (fused_moe.py:536).  Returns bf16 [T, H]."""
+    _need_gpu(rows, topk_w, src_to_dst)
+    T, K = topk_w.shape
+    H = rows.shape[1]
+    topk_w = topk_w.float().contiguous()
+    if init is not None:
+        init = init.to(torch.bfloat16).contiguous()
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=rows.device)
+    rc = L.lib().omni_moe_combine(_ptr(rows), _DT[rows.dtype], _ptr(topk_w), _ptr(src_to_dst), idx_mode, order, T, K, H,
+                                  _ptr(init), _ptr(post_add), _ptr(post_add_row0), _ptr(out), _stream())
+    L.check(rc, "omni_moe_combine")
+    return out
+
+
+def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: torch.Tensor, topk_ids: torch.Tensor,
+                   lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None, H: int = 0, I: int = 0,
+                   workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The whole local-share layer in one library call (quant if x is bf16, permute, GEMM1
+    epilogue, GEMM2, combine), the shared expert carried as an extra group."""
+    _need_gpu(x, topk_w, topk_ids)
+    T, K = topk_ids.shape
+    dev = x.device
+    x = x.contiguous()
+    topk_w = topk_w.float().contiguous()
+    topk_ids = topk_ids.to(torch.int32).contiguous()
+    x_dtype = -1 if x.dtype == torch.int8 else _DT[x.dtype]
+    sh = shared if shared is not None else (None, None, None, None)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, hi - lo, H, I, int(shared is not None))
+    if workspace is None or workspace.numel() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    rc = L.lib().omni_moe_w8a8_layer(_ptr(x), x_dtype, _ptr(x_scale), _ptr(topk_w), _ptr(topk_ids), T, K, lo, hi,
+                                     _ptr(w13_packed), _ptr(w13_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(sh[0]),
+                                     _ptr(sh[1]), _ptr(sh[2]), _ptr(sh[3]), H, I, _ptr(out), _ptr(workspace),
+                                     workspace.numel(), _stream())
+    L.check(rc, "omni_moe_w8a8_layer")
+    return out

@@ -1,0 +1,43 @@
+"""Replicated linear layers used by the MoE block: the gate and the shared expert's projections.
+
+Mirror of ``ReplicatedLinear`` / ``MergedReplicatedLinear`` as the MoE block uses them
+(omni/models/common/layers/linear.py:620-762; deepseek_moe.py:74-84,147-152): no tensor
+parallelism, ``forward`` returns ``(output, None)``.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+
+class ReplicatedLinear(nn.Module):
+    def __init__(self, input_size: int, output_size: int, bias: bool = False, quant_config=None,
+                 params_dtype: Optional[torch.dtype] = None, prefix: str = "", device=None):
+        super().__init__()
+        if bias:
+            raise NotImplementedError("bias is not used on the MoE path")
+        self.input_size, self.output_size = input_size, output_size
+        self.prefix = prefix
+        self.params_dtype = params_dtype or torch.get_default_dtype()
+        self.quant_method = quant_config.get_quant_method(self, prefix) if quant_config is not None else None
+        if self.quant_method is None:
+            self.weight = nn.Parameter(torch.empty(output_size, input_size, dtype=self.params_dtype, device=device),
+                                       requires_grad=False)
+        else:
+            self.quant_method.create_weights(self, [output_size], input_size, self.params_dtype, device=device)
+
+    def forward(self, x):
+        if self.quant_method is None:
+            return torch.nn.functional.linear(x, self.weight), None
+        return self.quant_method.apply_weights(self, x, None), None
+
+
+class MergedReplicatedLinear(ReplicatedLinear):
+    """gate_proj and up_proj stacked along the output dim (linear.py:620-762)."""
+
+    def __init__(self, input_size: int, output_sizes: List[int], bias: bool = False, quant_config=None,
+                 params_dtype: Optional[torch.dtype] = None, prefix: str = "", device=None):
+        self.output_sizes = output_sizes
+        super().__init__(input_size, sum(output_sizes), bias, quant_config, params_dtype, prefix, device)

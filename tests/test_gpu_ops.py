@@ -1,0 +1,229 @@
+"""Per-operator parity of the HIP kernels against the CPU oracle (bit exact), through the C ABI."""
+import os
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.helpers import Layer, gen, tokens
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from omni_infer_amd import hip_ops
+    return hip_ops
+
+
+def _eq(a, b, what):
+    a, b = a.cpu(), b.cpu()
+    assert a.shape == b.shape, f"{what}: shape {tuple(a.shape)} vs {tuple(b.shape)}"
+    if a.dtype.is_floating_point:
+        same = (a.view(torch.int32 if a.dtype == torch.float32 else torch.int16) ==
+                b.view(torch.int32 if b.dtype == torch.float32 else torch.int16)) | (a == b)
+    else:
+        same = a == b
+    bad = int((~same).sum())
+    assert bad == 0, f"{what}: {bad} of {a.numel()} elements differ; first at {torch.nonzero(~same)[0].tolist()}"
+
+
+# ------------------------------------------------------------------ routing
+@pytest.mark.parametrize("T,E,ng,tg,K", [(1, 256, 8, 4, 8), (64, 256, 8, 4, 8), (333, 256, 8, 4, 8),
+                                         (50, 64, 4, 2, 6), (17, 160, 8, 3, 6), (40, 384, 8, 4, 8)])
+def test_route_noaux_tc(ops, T, E, ng, tg, K):
+    g = gen(1)
+    logits = torch.randn(T, E, generator=g) * 2
+    bias = torch.randn(E, generator=g) * 0.01
+    w_ref, id_ref = O.route_noaux_tc(logits, bias, K, ng, tg, 2.5)
+    w, ids, _ = ops.npu_moe_gating_top_k(logits.cuda(), K, bias.cuda(), tg, ng, 1, 0, 1, 2.5, 1e-20)
+    _eq(ids, id_ref, "ids")
+    _eq(w, w_ref, "weights")
+
+
+def test_route_noaux_tc_ties(ops):
+    # many exactly equal logits: ties must go to the lower expert / group id
+    g = gen(2)
+    logits = torch.randint(-2, 3, (128, 256), generator=g).float()
+    bias = torch.zeros(256)
+    w_ref, id_ref = O.route_noaux_tc(logits, bias, 8, 8, 4, 2.5)
+    w, ids, _ = ops.npu_moe_gating_top_k(logits.cuda(), 8, bias.cuda(), 4, 8, 1, 0, 1, 2.5, 1e-20)
+    _eq(ids, id_ref, "ids")
+    _eq(w, w_ref, "weights")
+
+
+@pytest.mark.parametrize("scoring,with_bias", [("softmax", False), ("sigmoid", False), ("sigmoid", True)])
+def test_route_grouped_topk(ops, scoring, with_bias):
+    from omni_infer_amd.layers.fused_moe import grouped_topk
+    g = gen(3)
+    T, E = 97, 256
+    logits = torch.randn(T, E, generator=g)
+    bias = torch.randn(E, generator=g) * 0.01 if with_bias else None
+    w_ref, id_ref, row_ref = O.route_grouped_topk(logits, 8, True, 8, 4, scoring, bias)
+    w, ids, row = grouped_topk(None, logits.cuda(), 8, True, 8, 4, scoring, None if bias is None else bias.cuda())
+    _eq(ids, id_ref, "ids")
+    _eq(w, w_ref, "weights")
+    _eq(row.contiguous(), row_ref, "row_idx")
+
+
+@pytest.mark.parametrize("T,E,K,renorm", [(64, 8, 2, True), (64, 8, 2, False), (5, 64, 4, True), (33, 200, 6, True),
+                                          (9, 512, 8, True)])
+def test_route_softmax_topk(ops, T, E, K, renorm):
+    from omni_infer_amd.layers.fused_moe import fused_topk
+    logits = torch.randn(T, E, generator=gen(4)) * 3
+    w_ref, id_ref, row_ref = O.route_softmax_topk(logits, K, renorm)
+    w, ids, row = fused_topk(logits.cuda(), K, renorm)
+    _eq(ids, id_ref, "ids")
+    _eq(w, w_ref, "weights")
+    _eq(row.contiguous(), row_ref, "row_idx")
+
+
+# ------------------------------------------------------------------ dynamic quant
+@pytest.mark.parametrize("T,H,dtype", [(64, 7168, torch.bfloat16), (3, 7680, torch.bfloat16), (5, 1024, torch.bfloat16),
+                                       (7, 100, torch.bfloat16), (2, 16384, torch.bfloat16),
+                                       (6, 2048, torch.float32), (4, 520, torch.float16)])
+def test_dynamic_quant(ops, T, H, dtype):
+    x = (torch.randn(T, H, generator=gen(5)) * 3).to(dtype)
+    x[:, :: max(1, H // 7)] *= 50          # outlier channels
+    if T > 1:
+        x[1] = 0                             # an all-zero row
+    q_ref, s_ref = O.dynamic_quant(x)
+    q, s = ops.npu_dynamic_quant(x.cuda())
+    _eq(s, s_ref, "scale")
+    _eq(q, q_ref, "q")
+
+
+def test_dynamic_quant_strided_and_3d(ops):
+    x = torch.randn(4, 6, 512, generator=gen(6)).to(torch.bfloat16)
+    q_ref, s_ref = O.dynamic_quant(x)
+    q, s = ops.npu_dynamic_quant(x.cuda())
+    _eq(q, q_ref, "q")
+    _eq(s, s_ref, "scale")
+    big = torch.randn(8, 1024, generator=gen(7)).to(torch.bfloat16)
+    view = big[:, :512]                      # row stride 1024, 512 columns
+    q_ref, s_ref = O.dynamic_quant(view)
+    q, s = ops.npu_dynamic_quant(big.cuda()[:, :512])
+    _eq(q, q_ref, "q strided")
+    _eq(s, s_ref, "scale strided")
+
+
+# ------------------------------------------------------------------ permutation
+@pytest.mark.parametrize("T,K,E,lo,hi", [(64, 8, 256, 0, 32), (64, 8, 256, 96, 128), (1, 8, 256, 0, 32),
+                                         (500, 8, 256, 32, 64), (2048, 8, 256, 0, 32), (700, 6, 64, 0, 64),
+                                         (64, 2, 8, 0, 8), (1100, 8, 256, 0, 256)])
+def test_permute_v2(ops, T, K, E, lo, hi):
+    g = gen(8)
+    ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    x = torch.randint(-128, 128, (T, 64), generator=g, dtype=torch.int8)
+    sc = torch.rand(T, generator=g)
+    rows_ref, idx_ref, counts_ref, sc_ref = O.moe_init_routing_v2(x, ids, sc, (lo, hi))
+    rows, idx, counts, scg = ops.npu_moe_init_routing_v2(x.cuda(), ids.cuda(), scale=sc.cuda(),
+                                                         active_expert_range=[lo, hi], expert_num=E)
+    m = idx_ref.numel()
+    _eq(counts, counts_ref, "counts")
+    _eq(idx[:m], idx_ref, "expanded_x_idx")
+    _eq(rows[:m], rows_ref, "rows")
+    _eq(scg[:m], sc_ref, "scale")
+    # the tail holds the dropped assignments in their original order: still a permutation
+    assert sorted(idx.cpu().tolist()) == list(range(T * K))
+
+
+def test_permute_v1_and_empty(ops):
+    g = gen(9)
+    T, K, E = 200, 2, 8
+    ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    ids[ids == 3] = 5                        # expert 3 receives nothing (and 5 may repeat in a token)
+    x = torch.randn(T, 32, generator=g).to(torch.bfloat16)
+    row_idx = torch.arange(T * K, dtype=torch.int32).view(K, T).t().contiguous()
+    rows_ref, s2d_ref, sid_ref = O.moe_init_routing_v1(x, row_idx, ids)
+    rows, s2d, sid = ops.npu_moe_init_routing(x.cuda(), row_idx.cuda(), ids.cuda(), T, num_experts=E)
+    _eq(rows, rows_ref, "rows")
+    _eq(s2d, s2d_ref, "src_to_dst")
+    _eq(sid, sid_ref, "sorted ids")
+    cum = ops.npu_moe_compute_expert_tokens(sid, E)
+    _eq(cum, O.compute_expert_tokens(sid_ref, E).to(torch.int32), "cumulative tokens")
+
+
+def test_permute_all_dropped(ops):
+    ids = torch.full((16, 4), 200, dtype=torch.int32)
+    from omni_infer_amd import _lib as L
+    p = ops.moe_permute(ids.cuda(), 0, 32, L.OMNI_IDX_TOKEN_MAJOR)
+    assert int(p.counts.sum()) == 0 and int(p.offsets[-1]) == 0
+    assert bool((p.src_to_dst.cpu() == -1).all())
+
+
+# ------------------------------------------------------------------ weight packing
+@pytest.mark.parametrize("layout", [0, 1])
+def test_pack_weight_layout(ops, layout):
+    g = gen(10)
+    G, Kd, N = 2, 128, 48
+    w = torch.randint(-128, 128, (G, Kd, N), generator=g, dtype=torch.int8)      # logical [G, K, N]
+    src = w if layout == 0 else w.transpose(1, 2).contiguous()
+    packed = ops.pack_weight(src.cuda(), layout).cpu().view(G, -1)
+    k = torch.arange(Kd).view(-1, 1)
+    n = torch.arange(N).view(1, -1)
+    off = (((n // 16) * (Kd // 64) + k // 64) * 64 + (n % 16) + 16 * ((k % 64) // 16)) * 16 + k % 16
+    for gi in range(G):
+        assert bool((packed[gi][off.reshape(-1)] == w[gi].reshape(-1)).all())
+
+
+# ------------------------------------------------------------------ GEMM1 / GEMM2 / combine
+def _grouped_case(T, K, n_local, E, H, I, seed, lo=0):
+    g = gen(seed)
+    lay = Layer(n_local, H, I, seed)
+    x = tokens(T, H, seed + 1)
+    xq, xs = O.dynamic_quant(x)
+    ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    w = torch.rand(T, K, generator=g)
+    return lay, xq, xs, ids, w
+
+
+@pytest.mark.parametrize("T,K,n_local,E,H,I,force", [
+    (64, 2, 8, 8, 1024, 512, 0),        # toy shape, stream kernel
+    (64, 8, 4, 32, 7168, 2048, 0),      # DeepSeek-V3 widths, 4 local experts of 32
+    (16, 8, 4, 32, 7680, 2048, 0),      # Pangu widths
+    (300, 4, 4, 8, 1024, 512, 1),       # ragged groups > 64 rows through the stream kernel
+    (300, 4, 4, 8, 1024, 512, 2),       # same through the tile kernel
+    (1100, 4, 3, 6, 512, 256, 0),       # tile kernel by default, partial 256-row blocks
+])
+def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, monkeypatch):
+    from omni_infer_amd import _lib as L
+    if force:
+        monkeypatch.setenv("OMNI_MOE_FORCE_KERNEL", str(force))
+    lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 20 + T)
+    d = lay.to_device()
+    out_ref, st = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (0, n_local),
+                                                    return_stages=True)
+    p = ops.moe_permute(ids.cuda(), 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    m = int(st["counts"].sum())
+    M_cap = T * K
+    h_q, h_s, acc1 = ops.grouped_gemm1_swiglu_quant(xq.cuda(), xs.cuda(), p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K,
+                                                    d["w13"], d["s13"], p.offsets, H, I, M_cap, want_acc=True)
+    _eq(acc1[:m], st["acc1"], "GEMM1 int32 accumulators")
+    _eq(h_s[:m], st["h_s"], "stage-2 scales")
+    _eq(h_q[:m], st["h_q"], "stage-2 int8 activations")
+    for dt in (torch.float32, torch.bfloat16):
+        rows, acc2 = ops.grouped_gemm2_dequant(h_q, h_s, d["w2"], d["s2"], p.offsets, H, I, out_dtype=dt, want_acc=True)
+        _eq(acc2[:m], st["acc2"], "GEMM2 int32 accumulators")
+        g_of = torch.repeat_interleave(torch.arange(n_local), st["counts"])
+        ref_rows = ((st["acc2"].float() * lay.s2[g_of]) * st["h_s"].unsqueeze(-1)).to(dt)
+        _eq(rows[:m], ref_rows, f"GEMM2 rows {dt}")
+    rows32, _ = ops.grouped_gemm2_dequant(h_q, h_s, d["w2"], d["s2"], p.offsets, H, I, out_dtype=torch.float32)
+    out = ops.moe_combine(rows32, w.cuda(), p.src_to_dst, L.OMNI_IDX_TOKEN_MAJOR, L.OMNI_ORDER_SLOT)
+    _eq(out, out_ref, "combined output")
+
+
+def test_combine_k_order_with_skip(ops):
+    from omni_infer_amd import _lib as L
+    g = gen(30)
+    T, K, H, E = 50, 4, 256, 8
+    ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    w = torch.rand(T, K, generator=g)
+    rows = torch.randn(T * K, H, generator=g).to(torch.bfloat16)
+    skip = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    for mode, omode in ((0, L.OMNI_IDX_K_MAJOR), (2, L.OMNI_IDX_TOKEN_MAJOR)):
+        p = ops.moe_permute(ids.cuda(), 0, 6, omode)       # experts 6, 7 are not local: dropped rows
+        ref = O.moe_finalize_routing(rows.float(), skip, w, p.src_to_dst.cpu(), drop_pad_mode=mode).to(torch.bfloat16)
+        out = ops.moe_combine(rows.cuda(), w.cuda(), p.src_to_dst, omode, L.OMNI_ORDER_K, init=skip.cuda())
+        _eq(out, ref, f"finalize mode {mode}")
