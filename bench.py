@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 fused-MoE layer on one MI355X.
+
+A step is one pass of the layer over one batch of synthetic tokens, inputs resident in HBM:
+    router (sigmoid + bias, 8 groups / top-4, top-8)  ->  per-token int8 quantisation  ->
+    sort by expert  ->  int8 GEMM1 + dequant + SwiGLU + requant  ->  int8 GEMM2 + dequant  ->
+    weighted combine + shared expert.
+Workloads (BASELINE.json configs):
+    decode   DeepSeek-V3 shape, 32 local experts of 256 + 1 shared expert, 64 tokens   (default)
+    prefill  same layer, 8192 tokens with 0.1 % outlier channels x50
+Router logits are random over the 32 local experts and -30 elsewhere, so the router itself
+sends every token to 8 distinct local experts ("uniform random routing into local experts").
+The gate GEMM that makes the logits is not part of the step.
+
+Prints one JSON line: layer time, the roofline figure of the dominant kernel (GEMM1), and the
+CPU oracle timed on this box's host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12       # B/s, MI355X published
+INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/clk x 2.4 GHz = 5.03e15)
+
+SHAPES = {
+    "decode": dict(T=64, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5, outlier=0.0),
+    "prefill": dict(T=8192, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5,
+                    outlier=0.001),
+}
+
+
+def make_weights(n_local, H, I, seed, dev):
+    """fp32 N(0, 0.02) weights quantised to symmetric per-output-channel int8 (checkpoint layout)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+
+    def q(out_f, in_f):
+        w = torch.randn(out_f, in_f, generator=g, device=dev) * 0.02
+        s = w.abs().amax(dim=1) / 127.0
+        return torch.round(w / s.unsqueeze(1)).clamp(-127, 127).to(torch.int8), s
+
+    w13 = torch.empty(n_local, 2 * I, H, dtype=torch.int8, device=dev)
+    w2 = torch.empty(n_local, H, I, dtype=torch.int8, device=dev)
+    s13 = torch.empty(n_local, 2 * I, device=dev)
+    s2 = torch.empty(n_local, H, device=dev)
+    for e in range(n_local):
+        w13[e], s13[e] = q(2 * I, H)
+        w2[e], s2[e] = q(H, I)
+    return w13, s13, w2, s2
+
+
+class WeightSet:
+    def __init__(self, cfg, seed, dev):
+        from omni_infer_amd import hip_ops as ops
+        H, I, n = cfg["H"], cfg["I"], cfg["n_local"]
+        w13, self.s13, w2, self.s2 = make_weights(n, H, I, seed, dev)
+        sw13, ss13, sw2, ss2 = make_weights(1, H, I, seed + 1000, dev)
+        self.ckpt = (w13, w2, sw13[0], sw2[0])          # kept for the CPU baseline (set 0 only)
+        self.w13 = ops.pack_weight(w13, 1)
+        self.w2 = ops.pack_weight(w2, 1)
+        self.sh13 = ops.pack_weight(sw13[0], 1)
+        self.sh2 = ops.pack_weight(sw2[0], 1)
+        self.sh_s13, self.sh_s2 = ss13[0].contiguous(), ss2[0].contiguous()
+
+    def drop_ckpt(self):
+        self.ckpt = None
+
+
+def make_inputs(cfg, dev):
+    g = torch.Generator().manual_seed(0)
+    T, H, E, n_local = cfg["T"], cfg["H"], cfg["E"], cfg["n_local"]
+    x = torch.randn(T, H, generator=g)
+    if cfg["outlier"] > 0:
+        n = max(1, int(round(H * cfg["outlier"])))
+        ch = torch.randperm(H, generator=g)[:n]
+        x[:, ch] *= 50.0
+    logits = torch.full((T, E), -30.0)
+    logits[:, :n_local] = torch.randn(T, n_local, generator=g)
+    bias = torch.randn(E, generator=g) * 0.01
+    return x.to(torch.bfloat16).to(dev), logits.to(dev), bias.to(dev)
+
+
+def algorithmic_bytes_layer(cfg, groups_active):
+    H, I, T = cfg["H"], cfg["I"], cfg["T"]
+    w = groups_active * (H * 2 * I + I * H)
+    sc = groups_active * (2 * I + H) * 4
+    return w + sc + T * H * 2 + T * H * 2
+
+
+def algorithmic_ops_layer(cfg, rows_routed):
+    H, I, T = cfg["H"], cfg["I"], cfg["T"]
+    return 2 * (rows_routed + T) * (H * 2 * I + I * H)
+
+
+def cpu_baseline(cfg, ws, x, logits, bias, sample_tokens):
+    """The oracle's whole layer on the host cores, on the first `sample_tokens` tokens."""
+    from oracle import moe_oracle as O
+    torch.set_num_threads(os.cpu_count() or 1)
+    w13, w2, sw13, sw2 = [t.cpu() for t in ws.ckpt]
+    routed = (w13.transpose(1, 2).contiguous(), ws.s13.cpu(), w2.transpose(1, 2).contiguous(), ws.s2.cpu())
+    shared = (sw13.t().contiguous(), ws.sh_s13.cpu(), sw2.t().contiguous(), ws.sh_s2.cpu())
+    xs, ls, b = x[:sample_tokens].cpu(), logits[:sample_tokens].cpu(), bias.cpu()
+
+    def run():
+        return O.deepseek_moe_forward(xs, ls, b, routed, shared, cfg["K"], cfg["n_group"], cfg["topk_group"],
+                                      cfg["scale"], (0, cfg["n_local"]))
+    t0 = time.perf_counter()
+    out = run()
+    first = time.perf_counter() - t0
+    reps = 1 if first > 8.0 else 3
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        out = run()
+    dt = (time.perf_counter() - t0) / reps
+    return dt, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=sorted(SHAPES), default="decode")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--weight-sets", type=int, default=2, help="weight copies rotated between steps (cache defeat)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's expert share on one GPU; --gpus must be 1 "
+              "(no collectives are part of it)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+
+    cfg = SHAPES[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    T, H, I, K, n_local = cfg["T"], cfg["H"], cfg["I"], cfg["K"], cfg["n_local"]
+    if args.workload == "prefill" and args.steps == 200:
+        args.steps, args.warmup = 20, 3
+
+    sets = [WeightSet(cfg, 100 + i, dev) for i in range(max(1, args.weight_sets))]
+    for s in sets[1:]:
+        s.drop_ckpt()
+    x, logits, bias = make_inputs(cfg, dev)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, 1)
+    workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+
+    def step(i):
+        ws = sets[i % len(sets)]
+        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
+                                             cfg["scale"], 1e-20)
+        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
+                                  (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = e0.elapsed_time(e1) / args.steps
+    ms = max(ms, 0.0)
+
+    # routing actually produced (rows per local expert) for the byte / op counts
+    w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
+    p = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    counts = p.counts.cpu()
+    rows_routed = int(counts.sum())
+    active = int((counts > 0).sum()) + 1
+    layer_bytes = algorithmic_bytes_layer(cfg, active)
+    layer_ops = algorithmic_ops_layer(cfg, rows_routed)
+
+    # ---- dominant kernel alone: GEMM1 (one launch per call), timed with events on its stream
+    M_cap = T * K + T
+    xq, xs = ops.npu_dynamic_quant(x)
+    g1_ws = torch.zeros(L.lib().omni_moe_gemm1_workspace_bytes(M_cap, I), dtype=torch.uint8, device=dev)
+    hq = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
+    hs = torch.empty(M_cap, dtype=torch.float32, device=dev)
+    kflags = L.OMNI_GEMM1_NO_PROLOGUE | L.OMNI_GEMM1_NO_REQUANT
+
+    def gemm1_only(i):
+        ws = sets[i % len(sets)]
+        ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, ws.w13, ws.s13, p.offsets, H, I,
+                                       M_cap, extra=(ws.sh13, ws.sh_s13), extra_rows=T, flags=kflags, workspace=g1_ws,
+                                       out=(hq, hs))
+    ksteps = max(10, args.steps // 2)
+    for i in range(5):
+        gemm1_only(i)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(ksteps):
+        gemm1_only(i)
+    e1.record()
+    torch.cuda.synchronize()
+    k_ms = e0.elapsed_time(e1) / ksteps
+    rows_total = rows_routed + T
+    if args.workload == "decode":
+        k_alg = active * (H * 2 * I + 2 * I * 4) + T * H + T * 4 + rows_total * I * 4 + rows_total * 4
+        roof = dict(bound="hbm", kernel="gemm_stream<GEMM1>", achieved=k_alg / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9,
+                    unit="GB/s")
+    else:
+        k_alg = 2 * rows_total * H * 2 * I
+        roof = dict(bound="mfma", kernel="gemm_tile<GEMM1>", achieved=k_alg / (k_ms * 1e-3) / 1e12, peak=INT8_PEAK / 1e12,
+                    unit="TFLOP/s")
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_us"] = k_ms * 1e3
+    roof["algorithmic_per_launch"] = k_alg
+    roof["traffic"] = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            roof["traffic"] = json.load(f).get(args.workload)
+
+    result = {
+        "metric": "moe_layer_latency", "value": ms * 1e3, "unit": "us", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": f"DeepSeek-V3-shape W8A8 MoE layer, {args.workload}: {T} tokens, {n_local} local experts "
+                               f"of {cfg['E']} + 1 shared, H={H}, I={I}, top-{K} grouped sigmoid routing",
+                   "tokens": T, "rows_routed": rows_routed, "active_groups": active, "weight_sets": len(sets)},
+        "layer": {"algorithmic_bytes": layer_bytes, "algorithmic_ops": layer_ops,
+                  "hbm_frac": layer_bytes / (ms * 1e-3) / HBM_PEAK, "int8_frac": layer_ops / (ms * 1e-3) / INT8_PEAK,
+                  "host_wall_ms_per_step": wall_ms},
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        sample = T if args.workload == "decode" else 128
+        dt, ref = cpu_baseline(cfg, sets[0], x, logits, bias, sample)
+        got = step(0)[:sample].float().cpu()
+        torch.cuda.synchronize()
+        refd = ref.float()
+        rel = float((got - refd).norm() / refd.norm())
+        result["cpu_baseline"] = {"value": dt * 1e6 * (T / sample), "unit": "us", "cores": torch.get_num_threads(),
+                                  "kind": "port",
+                                  "sample": f"oracle layer on the first {sample} of {T} tokens "
+                                            f"({dt:.2f} s per pass" + (", scaled by tokens)" if sample != T else ")"),
+                                  "gpu_vs_oracle_rel_err": rel,
+                                  "gpu_vs_oracle_bit_exact": bool(torch.equal(got, refd))}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -56,6 +56,10 @@ extern "C" {
 /* gemm flags */
 #define OMNI_GEMM1_BF16_INTERMEDIATE 1 /* round the dequantised gate/up and the SwiGLU product to bf16
                                           (numerics of the non-EP pipeline, compressed_tensors_moe.py:242-247) */
+#define OMNI_GEMM1_NO_PROLOGUE 2  /* do not clear the row-maximum words first (the caller did) */
+#define OMNI_GEMM1_NO_REQUANT 4   /* stop after the GEMM kernel: y and the row maxima stay in the workspace,
+                                     h_q / h_scale are not written.  With NO_PROLOGUE the call is exactly one
+                                     kernel launch, which is how the benchmark times that kernel alone. */
 /* combine: how src_to_dst is indexed */
 #define OMNI_IDX_TOKEN_MAJOR 0 /* n*K + k  (npu_moe_init_routing_v2 row_idx_type=1; finalize drop_pad_mode=2) */
 #define OMNI_IDX_K_MAJOR 1     /* k*T + n  (npu_moe_init_routing; finalize drop_pad_mode=0) */
@@ -142,8 +146,8 @@ int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N
  *   Rows are grouped: group g owns rows [offsets[g], offsets[g+1]); an optional extra group
  *   (w13_extra != NULL) owns rows [offsets[G], offsets[G] + extra_rows) and maps row r to source
  *   row r - offsets[G] (the shared expert on every token).
- *   Row m of a regular group reads x_q[sorted_src[m] / src_div] (idx_mode TOKEN_MAJOR) or
- *   x_q[sorted_src[m] % src_mod] (K_MAJOR); sorted_src NULL: row m reads x_q[m].
+ *   Row m of a regular group reads x_q[sorted_src[m] / K] (idx_mode TOKEN_MAJOR) or
+ *   x_q[sorted_src[m] % T] (K_MAJOR); sorted_src NULL: row m reads x_q[m].
  *   acc = x_q[row] . W13[g]  (int32, exact);  d = (float(acc) * w13_scale[g][n]) * x_scale[row];
  *   y = silu(d[:I]) * d[I:];  h_scale[m] = max|y| / 127;  h_q = rint(y / h_scale).
  *   w13 packed: G matrices of Kdim = H, N = 2I (gate channels first).

@@ -35,7 +35,7 @@ SIGNATURES = {
 OMNI_DT_BF16, OMNI_DT_F32, OMNI_DT_F16 = 0, 1, 2
 OMNI_SCORE_SOFTMAX, OMNI_SCORE_SIGMOID = 0, 1
 OMNI_GROUP_MAX, OMNI_GROUP_TOP2SUM = 0, 1
-OMNI_GEMM1_BF16_INTERMEDIATE = 1
+OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_PROLOGUE, OMNI_GEMM1_NO_REQUANT = 1, 2, 4
 OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 
@@ -53,6 +53,10 @@ def lib() -> ctypes.CDLL:
             raise OmniMoeError(
                 f"{LIB_PATH} is missing: build it with `python -m omni_infer_amd._build` "
                 "(hipcc --offload-arch=gfx950); there is no fallback implementation")
+        # torch ships its own HIP runtime (same soname as /opt/rocm's).  The library must bind to
+        # the runtime torch initialised, or its launches would see another runtime's streams and
+        # devices: make sure torch is loaded first.
+        import torch  # noqa: F401
         handle = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)  # AttributeError if the library does not export it

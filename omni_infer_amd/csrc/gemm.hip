@@ -563,7 +563,8 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   hipStream_t st = (hipStream_t)stream;
   float* y = (float*)workspace;
   uint32_t* rowmax = (uint32_t*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
-  hipLaunchKernelGGL(zero_u32, dim3((unsigned)((M_cap + 255) / 256)), dim3(256), 0, st, rowmax, M_cap);
+  if (!(flags & OMNI_GEMM1_NO_PROLOGUE))
+    hipLaunchKernelGGL(zero_u32, dim3((unsigned)((M_cap + 255) / 256)), dim3(256), 0, st, rowmax, M_cap);
   GemmArgs a{};
   a.a_q = x_q; a.a_scale = x_scale; a.sorted_src = sorted_src; a.idx_mode = idx_mode; a.T = T; a.K = K;
   a.w = w13_packed; a.w_scale = w13_scale; a.w_extra = w13_extra; a.w_extra_scale = w13_extra_scale;
@@ -571,6 +572,7 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   a.y = y; a.rowmax = rowmax; a.acc_dbg = acc_dbg;
   rc = dispatch_gemm<1>(a, M_cap, st, "gemm1");
   if (rc) return rc;
+  if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
   hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax, offsets, G,
                      extra_rows, I, M_cap, h_q, h_scale);
   OMNI_CHECK_LAUNCH("gemm1 quant");

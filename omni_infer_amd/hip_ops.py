@@ -210,22 +210,27 @@ def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_
                                idx_mode: int, K: int, w13_packed: torch.Tensor, w13_scale: torch.Tensor,
                                offsets: torch.Tensor, H: int, I: int, M_cap: int,
                                extra: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, extra_rows: int = 0,
-                               bf16_intermediate: bool = False, want_acc: bool = False):
+                               bf16_intermediate: bool = False, want_acc: bool = False, flags: int = 0,
+                               workspace: Optional[torch.Tensor] = None, out=None):
     """GEMM1 + dequant + SwiGLU + requant: ``npu_grouped_matmul(int32)`` +
     ``npu_dequant_swiglu_quant`` (fused_moe.py:531-534, :670-677).  Returns (h_q, h_scale, acc)."""
     _need_gpu(x_q, x_scale, w13_packed, w13_scale, offsets)
     dev = x_q.device
     T = x_q.shape[0]
     G = offsets.numel() - 1
-    h_q = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
-    h_s = torch.empty(M_cap, dtype=torch.float32, device=dev)
+    if out is None:
+        h_q = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
+        h_s = torch.empty(M_cap, dtype=torch.float32, device=dev)
+    else:
+        h_q, h_s = out
     acc = torch.zeros(M_cap, 2 * I, dtype=torch.int32, device=dev) if want_acc else None
     ws_bytes = L.lib().omni_moe_gemm1_workspace_bytes(M_cap, I)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = workspace if workspace is not None else torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     ew, es = extra if extra is not None else (None, None)
     rc = L.lib().omni_moe_gemm1_swiglu_quant(
         _ptr(x_q), _ptr(x_scale), _ptr(sorted_src), idx_mode, T, K, _ptr(w13_packed), _ptr(w13_scale), _ptr(ew),
-        _ptr(es), extra_rows, _ptr(offsets), G, H, I, M_cap, L.OMNI_GEMM1_BF16_INTERMEDIATE if bf16_intermediate else 0,
+        _ptr(es), extra_rows, _ptr(offsets), G, H, I, M_cap,
+        flags | (L.OMNI_GEMM1_BF16_INTERMEDIATE if bf16_intermediate else 0),
         _ptr(h_q), _ptr(h_s), _ptr(acc), _ptr(ws), ws_bytes, _stream())
     L.check(rc, "omni_moe_gemm1_swiglu_quant")
     return h_q, h_s, acc
@@ -234,14 +239,14 @@ def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_
 def grouped_gemm2_dequant(h_q: torch.Tensor, h_scale: torch.Tensor, w2_packed: torch.Tensor, w2_scale: torch.Tensor,
                           offsets: torch.Tensor, H: int, I: int, out_dtype: torch.dtype = torch.bfloat16,
                           extra: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, extra_rows: int = 0,
-                          want_acc: bool = False):
+                          want_acc: bool = False, out: Optional[torch.Tensor] = None):
     """GEMM2 + dequant: ``npu_grouped_matmul(scale=, per_token_scale=, output_dtype=bf16)``
     (fused_moe.py:570-574, :681-685).  Returns (rows [M_cap, H], acc)."""
     _need_gpu(h_q, h_scale, w2_packed, w2_scale, offsets)
     dev = h_q.device
     M_cap = h_q.shape[0]
     G = offsets.numel() - 1
-    rows = torch.zeros(M_cap, H, dtype=out_dtype, device=dev)
+    rows = out if out is not None else torch.zeros(M_cap, H, dtype=out_dtype, device=dev)
     acc = torch.zeros(M_cap, H, dtype=torch.int32, device=dev) if want_acc else None
     ew, es = extra if extra is not None else (None, None)
     rc = L.lib().omni_moe_gemm2_dequant(_ptr(h_q), _ptr(h_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(ew), _ptr(es),
