@@ -38,7 +38,7 @@ class AscendCompressedTensorsConfig:
     def get_quant_method(self, layer: torch.nn.Module, prefix: str):
         from ..layers.layer import FusedMoE
         from ..layers.linear import ReplicatedLinear
-        if any(prefix.endswith(ig) or ig in prefix for ig in self.ignore):
+        if any(prefix == ig or prefix.split(".")[-1] == ig for ig in self.ignore):
             return None
         if isinstance(layer, FusedMoE):
             layer.num_bits = self.num_bits

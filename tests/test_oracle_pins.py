@@ -1,0 +1,302 @@
+"""Pins of the CPU oracle against evidence that does not come from the oracle's own formulas:
+library routines (torch, transformers' DeepseekV3TopkRouter, numpy), the reference's own pure-torch
+routing code restated side by side, closed-form invariants, brute force on tiny inputs, and an
+end-to-end dense witness in float64.  The reference holds no golden vector for this path, so these
+pins (and the fixtures under tests/golden, which freeze the oracle's outputs) are what parity rests on."""
+import itertools
+import os
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.helpers import Layer, cosine, gen, rel_err, tokens
+
+
+def ulp_diff(a, b):
+    ai = a.contiguous().view(torch.int32).long()
+    bi = b.contiguous().view(torch.int32).long()
+    ai = torch.where(ai < 0, -(ai & 0x7fffffff), ai)
+    bi = torch.where(bi < 0, -(bi & 0x7fffffff), bi)
+    return (ai - bi).abs()
+
+
+# ------------------------------------------------------------------ transcendental
+def test_exp_spec_against_libm():
+    x = torch.linspace(-86.9, 86.9, 1_000_001)
+    got = O.exp_spec(x)
+    want = torch.exp(x.double()).float()
+    assert int(ulp_diff(got, want).max()) <= 2
+    assert float(O.exp_spec(torch.tensor([0.0]))) == 1.0
+    assert bool((got[1:] >= got[:-1]).all()), "exp must be monotone"
+    # clamping: finite, positive, normal numbers at both ends
+    ends = O.exp_spec(torch.tensor([-1e4, -87.0, 87.0, 1e4, float("inf"), float("-inf")]))
+    assert bool(torch.isfinite(ends).all()) and bool((ends >= torch.finfo(torch.float32).tiny).all())
+
+
+def test_sigmoid_silu_spec_against_torch():
+    x = torch.cat([torch.linspace(-30, 30, 600_001), torch.randn(100_000, generator=gen(0)) * 4])
+    s = O.sigmoid_spec(x)
+    assert float((s.double() - torch.sigmoid(x.double())).abs().max()) < 1.5e-7
+    y = O.silu_spec(x)
+    ref = torch.nn.functional.silu(x.double())
+    assert float((y.double() - ref).abs().max()) < 2e-6
+    nz = ref.abs() > 1e-30
+    assert float(((y.double() - ref)[nz] / ref[nz]).abs().max()) < 4e-7      # ~3 ulp
+    assert float(O.silu_spec(torch.tensor([0.0]))) == 0.0
+    assert float(O.sigmoid_spec(torch.tensor([0.0]))) == 0.5
+
+
+# ------------------------------------------------------------------ routing
+def _hf_router(E, K, n_group, topk_group, scale, bias):
+    from transformers.models.deepseek_v3.modeling_deepseek_v3 import DeepseekV3TopkRouter
+    cfg = types.SimpleNamespace(num_experts_per_tok=K, num_local_experts=E, hidden_size=E, routed_scaling_factor=scale,
+                                n_group=n_group, topk_group=topk_group, norm_topk_prob=True)
+    r = DeepseekV3TopkRouter(cfg)
+    with torch.no_grad():
+        r.weight.copy_(torch.eye(E))            # logits = input, exactly
+        r.e_score_correction_bias.copy_(bias)
+    return r
+
+
+@pytest.mark.parametrize("T,E,ng,tg,K", [(512, 256, 8, 4, 8), (64, 64, 4, 2, 6), (33, 32, 8, 4, 8)])
+def test_route_noaux_tc_against_transformers(T, E, ng, tg, K):
+    g = gen(1)
+    logits = torch.randn(T, E, generator=g) * 2
+    bias = torch.randn(E, generator=g) * 0.01
+    w, ids = O.route_noaux_tc(logits, bias, K, ng, tg, 2.5)
+    with torch.no_grad():
+        lg, hw, hi = _hf_router(E, K, ng, tg, 2.5, bias)(logits)
+    assert torch.equal(lg, logits)
+    dense = torch.zeros(T, E).scatter_(1, ids.long(), w)
+    hdense = torch.zeros(T, E).scatter_(1, hi, hw)
+    assert bool(((dense != 0) == (hdense != 0)).all()), "selected expert sets differ from the library router"
+    assert float((dense - hdense).abs().max()) < 1e-6
+    # invariants
+    assert all(len(set(r.tolist())) == K for r in ids)
+    groups = ids // (E // ng)
+    assert all(len(set(r.tolist())) <= tg for r in groups)
+    assert float((w.sum(-1) - 2.5).abs().max()) < 1e-5
+    c = torch.sigmoid(logits) + bias
+    picked = torch.gather(c, 1, ids.long())
+    assert bool((picked[:, :-1] >= picked[:, 1:] - 1e-7).all()), "output must be in descending score"
+
+
+def test_route_noaux_tc_bruteforce_tiny():
+    """E=8, 4 groups of 2, keep 2 groups, top-2: enumerate every pair of groups and of experts."""
+    g = gen(2)
+    logits = torch.randn(200, 8, generator=g)
+    bias = torch.randn(8, generator=g) * 0.1
+    w, ids = O.route_noaux_tc(logits, bias, 2, 4, 2, 1.0)
+    s = O.sigmoid_spec(logits)
+    c = (s + bias).tolist()
+    for t in range(200):
+        gs = [c[t][2 * i] + c[t][2 * i + 1] for i in range(4)]
+        best_groups = max(itertools.combinations(range(4), 2), key=lambda p: (gs[p[0]] + gs[p[1]], -p[0], -p[1]))
+        cand = [2 * gi + j for gi in best_groups for j in range(2)]
+        best = sorted(cand, key=lambda e: (-c[t][e], e))[:2]
+        assert ids[t].tolist() == best
+
+
+def _reference_grouped_topk(gating_output, topk, renormalize, num_expert_group, topk_group, scoring_func, bias):
+    """fused_moe.py:38-84 restated line by line with torch's own softmax / sigmoid / topk."""
+    gating_output = gating_output.float()
+    scores = torch.softmax(gating_output, dim=-1) if scoring_func == "softmax" else gating_output.sigmoid()
+    if bias is not None:
+        scores = scores + bias.unsqueeze(0)
+    num_token = scores.shape[0]
+    group_scores = scores.view(num_token, num_expert_group, -1).max(dim=-1).values
+    group_idx = torch.topk(group_scores, k=topk_group, dim=-1, sorted=False)[1]
+    group_mask = torch.zeros_like(group_scores)
+    group_mask.scatter_(1, group_idx, 1)
+    score_mask = group_mask.unsqueeze(-1).expand(num_token, num_expert_group,
+                                                 scores.shape[-1] // num_expert_group).reshape(num_token, -1)
+    tmp_scores = scores.masked_fill(~score_mask.bool(), 0.0)
+    topk_weights, topk_ids = torch.topk(tmp_scores, k=topk, dim=-1, sorted=False)
+    if renormalize:
+        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+    return topk_weights, topk_ids.int()
+
+
+@pytest.mark.parametrize("scoring,with_bias", [("softmax", False), ("sigmoid", False), ("sigmoid", True)])
+def test_route_grouped_topk_against_reference_torch_code(scoring, with_bias):
+    g = gen(3)
+    logits = torch.randn(300, 256, generator=g)
+    bias = torch.randn(256, generator=g) * 0.01 if with_bias else None
+    w, ids, row = O.route_grouped_topk(logits, 8, True, 8, 4, scoring, bias)
+    rw, rid = _reference_grouped_topk(logits, 8, True, 8, 4, scoring, bias)
+    a = torch.zeros(300, 256).scatter_(1, ids.long(), w)
+    b = torch.zeros(300, 256).scatter_(1, rid.long(), rw)
+    assert bool(((a != 0) == (b != 0)).all())
+    assert float((a - b).abs().max()) < 1e-6
+    assert row[5, 3] == 3 * 300 + 5
+
+
+def test_route_softmax_topk_against_torch():
+    logits = torch.randn(128, 8, generator=gen(4)) * 3
+    for renorm in (True, False):
+        w, ids, row = O.route_softmax_topk(logits, 2, renorm)
+        p = torch.softmax(logits, -1)
+        tw, ti = p.topk(2)
+        if renorm:
+            tw = tw / tw.sum(-1, keepdim=True)
+        assert torch.equal(ids.long(), ti)
+        assert float((w - tw).abs().max()) < 3e-7
+    assert float((O.softmax_spec(torch.randn(7, 300, generator=gen(5))).sum(-1) - 1).abs().max()) < 1e-6
+
+
+# ------------------------------------------------------------------ dynamic quant
+def test_dynamic_quant_invariants_and_numpy():
+    x = tokens(64, 7168, 6, outlier_frac=0.001)
+    x[3] = 0
+    q, s = O.dynamic_quant(x)
+    xf = x.float()
+    nz = s > 0
+    assert int(q[3].abs().max()) == 0 and float(s[3]) == 0.0
+    assert bool((q[nz].abs().amax(dim=1) == 127).all())
+    assert bool(((xf - q.float() * s.unsqueeze(1)).abs() <= s.unsqueeze(1) * 0.5 * (1 + 1e-6)).all())
+    # float32 numpy recomputation with a true division and round-half-even
+    xn = xf.numpy()
+    sn = (np.abs(xn).max(axis=1) / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        qn = np.where(sn[:, None] > 0, np.rint(xn / np.where(sn > 0, sn, 1)[:, None]), 0).clip(-128, 127)
+    assert np.array_equal(sn, s.numpy()) and np.array_equal(qn.astype(np.int8), q.numpy())
+    # idempotence: quantising the dequantised tensor gives the same integers
+    q2, s2 = O.dynamic_quant(q.float() * s.unsqueeze(1))
+    assert torch.equal(q2, q)
+    # half-way cases round to even
+    h = torch.tensor([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5]])
+    assert O.dynamic_quant(h)[0].tolist() == [[127, 0, 2, 2, 0, -2]]
+
+
+# ------------------------------------------------------------------ permutation
+def test_init_routing_v2_invariants():
+    g = gen(7)
+    T, K, E, lo, hi = 300, 8, 256, 64, 96
+    ids = torch.rand(T, E, generator=g).argsort(1)[:, :K].int()
+    x = torch.randint(-128, 128, (T, 16), generator=g, dtype=torch.int8)
+    sc = torch.rand(T, generator=g)
+    rows, idx, counts, scg = O.moe_init_routing_v2(x, ids, sc, (lo, hi))
+    flat = ids.reshape(-1).numpy()
+    keep = (flat >= lo) & (flat < hi)
+    order = np.argsort(np.where(keep, flat, 1 << 30), kind="stable")[:keep.sum()]
+    assert np.array_equal(idx.numpy(), order)
+    assert np.array_equal(counts.numpy(), np.bincount(flat[keep] - lo, minlength=hi - lo))
+    e_sorted = flat[idx.numpy()]
+    assert bool((np.diff(e_sorted) >= 0).all())
+    assert torch.equal(rows, x[idx.long() // K]) and torch.equal(scg, sc[idx.long() // K])
+
+
+def test_init_routing_v1_roundtrip():
+    g = gen(8)
+    T, K, E = 100, 2, 8
+    ids = torch.rand(T, E, generator=g).argsort(1)[:, :K].int()
+    x = torch.randn(T, 8, generator=g)
+    row_idx = torch.arange(T * K, dtype=torch.int32).view(K, T).t().contiguous()
+    rows, s2d, sid = O.moe_init_routing_v1(x, row_idx, ids)
+    assert sorted(s2d.tolist()) == list(range(T * K))
+    for n in (0, 17, 99):
+        for k in range(K):
+            d = int(s2d[k * T + n])
+            assert torch.equal(rows[d], x[n]) and int(sid[d]) == int(ids[n, k])
+    assert O.compute_expert_tokens(sid, E).tolist() == np.cumsum(np.bincount(ids.reshape(-1).numpy(), minlength=E)).tolist()
+
+
+# ------------------------------------------------------------------ GEMMs, epilogues, combine
+def test_grouped_matmul_int32_against_fp64():
+    g = gen(9)
+    a = torch.randint(-128, 128, (40, 7168), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (3, 7168, 64), generator=g, dtype=torch.int8)
+    counts = torch.tensor([17, 0, 23])
+    acc = O.grouped_matmul_int32(a, w, counts)
+    ref = torch.cat([a[:17].double() @ w[0].double(), a[17:].double() @ w[2].double()])
+    assert torch.equal(acc.double(), ref)
+    assert int(acc.abs().max()) < 2 ** 31
+
+
+def test_dequant_swiglu_quant_closed_form():
+    g = gen(10)
+    acc = torch.randint(-200000, 200000, (50, 256), generator=g, dtype=torch.int32)
+    ws = torch.rand(2, 256, generator=g) * 1e-3
+    ts = torch.rand(50, generator=g) * 0.05
+    counts = torch.tensor([20, 30])
+    q, s, y = O.dequant_swiglu_quant(acc, ws, ts, counts, return_fp32=True)
+    grp = torch.repeat_interleave(torch.arange(2), counts)
+    d = acc.double() * ws.double()[grp] * ts.double().unsqueeze(1)
+    yd = d[:, :128] / (1 + torch.exp(-d[:, :128])) * d[:, 128:]
+    assert rel_err(y, yd) < 1e-6
+    assert float((s.double() - yd.abs().amax(1) / 127).abs().max() / s.max()) < 1e-6
+    # gate is the first half, up the second: swapping halves must change the result
+    acc_sw = torch.cat([acc[:, 128:], acc[:, :128]], 1)
+    ws_sw = torch.cat([ws[:, 128:], ws[:, :128]], 1)
+    y_sw = O.dequant_swiglu_quant(acc_sw, ws_sw, ts, counts, return_fp32=True)[2]
+    assert not torch.allclose(y, y_sw)
+    # group_index=None form (dense linear) equals a single group
+    q1, s1 = O.dequant_swiglu_quant(acc, ws[0], ts, None)
+    q2, s2 = O.dequant_swiglu_quant(acc, ws[:1], ts, torch.tensor([50]))
+    assert torch.equal(q1, q2) and torch.equal(s1, s2)
+
+
+def test_finalize_routing_forms():
+    g = gen(11)
+    T, K, H = 20, 3, 32
+    rows = torch.randn(T * K, H, generator=g)
+    w = torch.rand(T, K, generator=g)
+    skip = torch.randn(T, H, generator=g)
+    s2d = torch.randperm(T * K, generator=g).int()
+    out0 = O.moe_finalize_routing(rows, skip, w, s2d, 0)
+    out2 = O.moe_finalize_routing(rows, skip, w, s2d, 2)
+    n = torch.arange(T)
+    ref0 = skip.double() + sum(w[:, k].double().unsqueeze(1) * rows[s2d[k * T + n].long()].double() for k in range(K))
+    ref2 = skip.double() + sum(w[:, k].double().unsqueeze(1) * rows[s2d[n * K + k].long()].double() for k in range(K))
+    assert rel_err(out0, ref0) < 1e-6 and rel_err(out2, ref2) < 1e-6
+    assert not torch.allclose(out0, out2)
+
+
+@pytest.mark.parametrize("T,K,n_local,E,H,I", [(64, 2, 8, 8, 1024, 512), (40, 8, 4, 32, 512, 256)])
+def test_pipeline_against_dense_bruteforce(T, K, n_local, E, H, I):
+    """The sorted / grouped / scattered pipeline equals the permutation-free dense computation."""
+    lay = Layer(n_local, H, I, seed=12)
+    g = gen(13)
+    x = tokens(T, H, 13)
+    xq, xs = O.dynamic_quant(x)
+    ids = torch.rand(T, E, generator=g).argsort(1)[:, :K].int()
+    w = torch.rand(T, K, generator=g)
+    lo = 0 if E == n_local else 8
+    out, st = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (lo, lo + n_local),
+                                                return_stages=True)
+    brute = O.dense_bruteforce(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (lo, lo + n_local))
+    assert rel_err(st["out32"], brute) < 2e-3          # int8 rounding flips between fp32 and fp64 SwiGLU
+    assert rel_err(out.float(), brute) < 5e-3
+    # and the non-EP pipeline (bf16 between stages) stays close to the same dense result
+    if E == n_local:
+        row_idx = torch.arange(T * K, dtype=torch.int32).view(K, T).t().contiguous()
+        out_u = O.fused_experts_w8a8(x, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, row_idx)
+        assert rel_err(out_u.float(), brute) < 2e-2
+
+
+def test_shared_expert_against_float_mlp():
+    lay = Layer(1, 1024, 512, seed=14, shared=True)
+    x = tokens(32, 1024, 14)
+    out = O.shared_expert_mlp(x, *lay.shared)
+    wgu = lay.shared[0].double() * lay.shared[1].double().unsqueeze(0)
+    wd = lay.shared[2].double() * lay.shared[3].double().unsqueeze(0)
+    h = x.double() @ wgu
+    y = torch.nn.functional.silu(h[:, :512]) * h[:, 512:]
+    assert rel_err(out.float(), y @ wd) < 4e-2           # noise of two int8 quantisations of the activations
+    assert cosine(out.float(), y @ wd) > 0.999
+
+
+# ------------------------------------------------------------------ golden fixtures
+def test_golden_fixtures_reproduce():
+    """tests/golden/*.pt freeze the oracle's outputs on the toy configuration (made by
+    tests/golden/make_golden.py); a change of the oracle's arithmetic shows up here."""
+    from tests.golden import make_golden
+    path = os.path.join(os.path.dirname(__file__), "golden", "toy_config1.pt")
+    saved = torch.load(path, weights_only=True)
+    fresh = make_golden.toy_config1()
+    assert sorted(saved) == sorted(fresh)
+    for k in saved:
+        assert torch.equal(saved[k], fresh[k]), k
