@@ -191,7 +191,7 @@ def main():
     # ---- dominant kernel alone: GEMM1 (one launch per call), timed with events on its stream
     M_cap = T * K + T
     xq, xs = ops.npu_dynamic_quant(x)
-    g1_ws = torch.zeros(L.lib().omni_moe_gemm1_workspace_bytes(M_cap, I), dtype=torch.uint8, device=dev)
+    g1_ws = torch.zeros(L.lib().omni_moe_gemm1_workspace_bytes(T, K, n_local, T, M_cap, H, I), dtype=torch.uint8, device=dev)
     hq = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
     hs = torch.empty(M_cap, dtype=torch.float32, device=dev)
     kflags = L.OMNI_GEMM1_NO_PROLOGUE | L.OMNI_GEMM1_NO_REQUANT
@@ -213,7 +213,8 @@ def main():
     k_ms = e0.elapsed_time(e1) / ksteps
     rows_total = rows_routed + T
     if args.workload == "decode":
-        k_alg = active * (H * 2 * I + 2 * I * 4) + T * H + T * 4 + rows_total * I * 4 + rows_total * 4
+        # weights of every active group + the int8 tokens + the int32 accumulators the kernel writes
+        k_alg = active * (H * 2 * I) + T * H + rows_total * 2 * I * 4
         roof = dict(bound="hbm", kernel="gemm_stream<GEMM1>", achieved=k_alg / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9,
                     unit="GB/s")
     else:

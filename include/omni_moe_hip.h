@@ -152,14 +152,14 @@ int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N
  *   y = silu(d[:I]) * d[I:];  h_scale[m] = max|y| / 127;  h_q = rint(y / h_scale).
  *   w13 packed: G matrices of Kdim = H, N = 2I (gate channels first).
  *   acc_dbg (nullable) [M_cap, 2I] receives the int32 accumulators.
- *   workspace: omni_moe_gemm1_workspace_bytes(M_cap, I).
+ *   workspace: omni_moe_gemm1_workspace_bytes(T, K, G, extra_rows, M_cap, H, I) (same arguments as the call).
  */
 int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode,
                                 int T, int K, const int8_t* w13_packed, const float* w13_scale,
                                 const int8_t* w13_extra, const float* w13_extra_scale, int extra_rows,
                                 const int32_t* offsets, int G, int H, int I, int64_t M_cap, int flags, int8_t* h_q,
                                 float* h_scale, int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream);
-size_t omni_moe_gemm1_workspace_bytes(int64_t M_cap, int I);
+size_t omni_moe_gemm1_workspace_bytes(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I);
 
 /*
  * GEMM2 + dequant.  Replaces npu_grouped_matmul(scale=, per_token_scale=, output_dtype=bf16)

@@ -168,7 +168,7 @@ LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
   L.perm_ws = take(L.perm_bytes);
   L.h_q = take((size_t)L.M_cap * I);
   L.h_s = take((size_t)L.M_cap * 4);
-  L.g1_bytes = omni_moe_gemm1_workspace_bytes(L.M_cap, I);
+  L.g1_bytes = omni_moe_gemm1_workspace_bytes(T, K, G, with_shared ? T : 0, L.M_cap, H, I);
   L.g1_ws = take(L.g1_bytes);
   L.rows = take((size_t)L.M_cap * H * 4);
   L.total = o;

@@ -49,6 +49,9 @@ struct GemmArgs {
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
   int32_t* acc_dbg;    // [M_cap, N], nullable
+  int32_t* part;       // GEMM1 stream kernel: [S, M_cap, N] partial accumulators (split-k)
+  int S;               // number of k splits (grid.z)
+  int64_t M_cap;
 };
 
 // source row of sorted row r of group g
@@ -122,11 +125,19 @@ __device__ __forceinline__ void flush_rowmax(const GemmArgs& a, int row0, int rb
 //   KIND 1: a wavefront owns NT (gate, up) strip pairs; KIND 2: NT strips.
 //   MT: 16-row tiles per block (block covers up to 16*MT rows of one group).
 //   D : k-steps of B kept in flight per wavefront (multiple of 4).
+//   Requires Kdim % (64*D) == 0 (checked on the host).
+//
+// The k loop is free of data-dependent branches: rows past the end of a group read the group's
+// first row (their accumulators are never stored), every tile of the block is multiplied, and
+// the loop is split into a part that refills the ring and a drain part, so the compiler can
+// count outstanding loads exactly and never waits for more than the oldest k-step.
 // =====================================================================================
 template <int KIND, int MT, int NT, int D>
 __global__ __launch_bounds__(256) void gemm_stream(GemmArgs a) {
   constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
   constexpr int BM = 16 * MT;
+  constexpr int DC = D / 4;                       // chunks (4 k-steps) of B in flight
+  static_assert(D % 4 == 0, "D counts whole chunks");
   __shared__ v4i lds_a[2][MT * 4 * WAVE];
 
   const int lane = threadIdx.x & (WAVE - 1);
@@ -135,7 +146,10 @@ __global__ __launch_bounds__(256) void gemm_stream(GemmArgs a) {
   if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, blockIdx.y, rb)) return;
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int mt_cnt = (nrows + 15) / 16;
-  const int nk64 = a.Kdim / 64;
+  const int nk64_all = a.Kdim / 64;          // k-steps of the whole reduction
+  const int nk64 = nk64_all / a.S;           // k-steps of this block's share
+  const int k64_0 = blockIdx.z * nk64;
+  const int nchunks = nk64 / 4;
   const int I = (KIND == 1) ? a.N / 2 : 0;
 
   const int8_t* wbase = (g < a.G) ? a.w + (size_t)g * a.Kdim * a.N : a.w_extra;
@@ -155,15 +169,16 @@ __global__ __launch_bounds__(256) void gemm_stream(GemmArgs a) {
     }
   }
 #pragma unroll
-  for (int j = 0; j < NBF; ++j) bp[j] = wbase + (size_t)strip[j] * nk64 * 1024 + lane * 16;
+  for (int j = 0; j < NBF; ++j) bp[j] = wbase + ((size_t)strip[j] * nk64_all + k64_0) * 1024 + lane * 16;
 
-  // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile
+  // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile, k-step w of
+  // every chunk; rows past the end of the group alias the group's first row
   const int8_t* arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     int rr = mt * 16 + (lane & 15);
-    arow[mt] = nullptr;
-    if (rr < nrows) arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (lane >> 4) * 16;
+    if (rr >= nrows) rr = 0;
+    arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k64_0 * 64 + (lane >> 4) * 16 + w * 64;
   }
 
   v4i acc[MT][NBF];
@@ -174,88 +189,161 @@ __global__ __launch_bounds__(256) void gemm_stream(GemmArgs a) {
 
   // ---- prologue: A chunk 0 -> LDS, first D k-steps of B -> ring
   v4i areg[MT];
-  {
-    const int ks = w;  // wavefront w stages k-step 4c + w of every chunk c
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      areg[mt] = (v4i){0, 0, 0, 0};
-      if (ks < nk64 && arow[mt]) areg[mt] = *(const v4i*)(arow[mt] + (size_t)ks * 64);
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) lds_a[0][(mt * 4 + w) * WAVE + lane] = areg[mt];
-  }
+  for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt]);
   v4i ring[D][NBF];
 #pragma unroll
   for (int s = 0; s < D; ++s)
 #pragma unroll
-    for (int j = 0; j < NBF; ++j) {
-      ring[s][j] = (v4i){0, 0, 0, 0};
-      if (s < nk64) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
-    }
+    for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) lds_a[0][(mt * 4 + w) * WAVE + lane] = areg[mt];
   __syncthreads();
 
-  for (int step = 0; step < nk64; step += D) {
+  // one chunk = 4 k-steps on ring slots [4*cc, 4*cc+4)
+  auto chunk = [&](const int c, const int cc, const bool refill) {
+    const int cnext = (c + 1 < nchunks) ? c + 1 : c;
 #pragma unroll
-    for (int s = 0; s < D; ++s) {
-      const int st = step + s;
-      if (st < nk64) {
-        const int c = st >> 2;
-        const int kk = s & 3;
-        if (kk == 0) {
-          // fetch this wavefront's share of the next A chunk while this one is consumed
-          const int ks = (c + 1) * 4 + w;
+    for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt] + (size_t)cnext * 256);
+    // keep these loads ahead of the ring refills below: they are waited for at the end of the
+    // chunk, and loads complete in order, so a later position would drain the whole ring
+    __builtin_amdgcn_sched_barrier(0);
+    const v4i* la = lds_a[c & 1];
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            areg[mt] = (v4i){0, 0, 0, 0};
-            if (ks < nk64 && arow[mt]) areg[mt] = *(const v4i*)(arow[mt] + (size_t)ks * 64);
-          }
-        }
-        v4i b[NBF];
+    for (int kk = 0; kk < 4; ++kk) {
+      const int s = cc * 4 + kk;
 #pragma unroll
-        for (int j = 0; j < NBF; ++j) {
-          b[j] = ring[s][j];
-          if (st + D < nk64) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)(st + D) * 1024));
-        }
+      for (int mt = 0; mt < MT; ++mt) {
+        v4i af = la[(mt * 4 + kk) * WAVE + lane];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          if (mt < mt_cnt) {
-            v4i af = lds_a[c & 1][(mt * 4 + kk) * WAVE + lane];
-#pragma unroll
-            for (int j = 0; j < NBF; ++j) acc[mt][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b[j], acc[mt][j], 0, 0, 0);
-          }
-        }
-        if (kk == 3 && st + 1 < nk64) {
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) lds_a[(c + 1) & 1][(mt * 4 + w) * WAVE + lane] = areg[mt];
-          __syncthreads();
-        }
+        for (int j = 0; j < NBF; ++j) acc[mt][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, ring[s][j], acc[mt][j], 0, 0, 0);
       }
+      // the slot is free once its MFMAs are issued: refill it with the k-step D ahead
+      if (refill) {
+#pragma unroll
+        for (int j = 0; j < NBF; ++j)
+          ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)(c * 4 + kk + D) * 1024));
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one k-step at a time: refills stay spread over the chunk
     }
+    v4i* ln = lds_a[(c + 1) & 1];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) ln[(mt * 4 + w) * WAVE + lane] = areg[mt];
+    __syncthreads();
+  };
+
+  int c0 = 0;
+  for (; c0 < nchunks - DC; c0 += DC) {
+#pragma unroll
+    for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, true);
   }
+#pragma unroll
+  for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, false);
 
   // ---- epilogue
   const int col = lane & 15;
+  if constexpr (KIND == 1) {
+    // raw int32 partial sums of this k share; the row kernel adds the shares and finishes
+    int32_t* part = a.part + (size_t)blockIdx.z * a.M_cap * a.N;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    if (mt < mt_cnt) {
-      const int rbase = mt * 16 + 4 * (lane >> 4);
-      float ts[4];
+    for (int mt = 0; mt < MT; ++mt) {
+      if (mt < mt_cnt) {
+        const int rbase = mt * 16 + 4 * (lane >> 4);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int rr = rbase + i;
-        ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
+        for (int j = 0; j < NBF; ++j) {
+          const int n = strip[j] * 16 + col;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (rbase + i < nrows) part[(size_t)(row0 + rbase + i) * a.N + n] = acc[mt][j][i];
+        }
       }
-      if constexpr (KIND == 1) {
-        float rmax[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    }
+  } else {
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          epilogue_gemm1(a, g, wsc, I, strip[2 * t] * 16 + col, row0, rbase, nrows, ts, acc[mt][2 * t], acc[mt][2 * t + 1], rmax);
-        flush_rowmax(a, row0, rbase, nrows, rmax);
-      } else {
+    for (int mt = 0; mt < MT; ++mt) {
+      if (mt < mt_cnt) {
+        const int rbase = mt * 16 + 4 * (lane >> 4);
+        float ts[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int rr = rbase + i;
+          ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsc, strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
       }
     }
+  }
+}
+
+// =====================================================================================
+// Row kernel after the split-k GEMM1: one 256-thread block per sorted row.  Adds the S partial
+// accumulators (exact in int32), dequantises, applies SwiGLU, reduces max|y| over the row and
+// quantises.  Each thread keeps its y values in registers between the two passes (PMAX pairs,
+// I <= 256*PMAX); nothing but the int8 row and its scale is written.
+// =====================================================================================
+template <int PMAX>
+__global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __restrict__ hq, float* __restrict__ hs) {
+  __shared__ float red[4];
+  __shared__ int s_group;
+  const int64_t m = blockIdx.x;
+  const int64_t total = (int64_t)a.offsets[a.G] + a.extra_rows;
+  if (m >= total) return;
+  if (threadIdx.x == 0) {
+    int lo = 0, hi = a.G;  // group g with offsets[g] <= m < offsets[g+1]; rows past offsets[G]: extra group
+    if (m >= a.offsets[a.G]) lo = a.G;
+    else {
+      while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (a.offsets[mid] <= m) lo = mid; else hi = mid;
+      }
+    }
+    s_group = lo;
+  }
+  __syncthreads();
+  const int g = s_group;
+  const int I = a.N / 2;
+  const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
+  const float ts = a.a_scale[source_row<1>(a, g, (int)m)];
+  const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+  const size_t plane = (size_t)a.M_cap * a.N;
+  const int32_t* prow = a.part + (size_t)m * a.N;
+  float y[PMAX];
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i) {
+    const int n = threadIdx.x + i * 256;
+    y[i] = 0.0f;
+    if (n < I) {
+      int ag = 0, au = 0;
+      for (int sp = 0; sp < a.S; ++sp) {
+        ag += prow[sp * plane + n];
+        au += prow[sp * plane + I + n];
+      }
+      if (a.acc_dbg) {
+        a.acc_dbg[(size_t)m * a.N + n] = ag;
+        a.acc_dbg[(size_t)m * a.N + I + n] = au;
+      }
+      float dg = ((float)ag * wsc[n]) * ts;
+      float du = ((float)au * wsc[I + n]) * ts;
+      if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+      float yv = silu_spec(dg) * du;
+      if (bf) yv = round_bf16(yv);
+      y[i] = yv;
+      amax = fmaxf(amax, fabsf(yv));
+    }
+  }
+  amax = wave_allmax_f(amax);
+  if ((threadIdx.x & (WAVE - 1)) == 0) red[threadIdx.x / WAVE] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float sc = amax / 127.0f;
+  if (threadIdx.x == 0) hs[m] = sc;
+  int8_t* qr = hq + (size_t)m * I;
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i) {
+    const int n = threadIdx.x + i * 256;
+    if (n < I) qr[n] = (sc > 0.0f) ? (int8_t)quant_i8(y[i], sc) : (int8_t)0;
   }
 }
 
@@ -447,21 +535,58 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(const int8_t* __restri
 // ---------------------------------------------------------------- host side dispatch
 struct Plan {
   bool tile;
-  int mt, nt;  // stream kernel parameters
+  int mt, nt, d;  // stream kernel parameters
+  int S;          // k splits (GEMM1 stream kernel only)
 };
 
-Plan choose_plan(int kind, int T, int K, int G, int extra_rows, int N_strips_unit) {
-  // expected rows of a busy group
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : dflt;
+}
+
+// Decides the kernel from what the host knows: the expected rows of a busy group.  The stream
+// kernel covers a group with blocks of 16*mt rows; GEMM1 is also split along k so that the
+// launch has several times more blocks than the chip has block slots (no idle tail).
+template <int KIND>
+Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_cap) {
+  const int units = (KIND == 1) ? N / 32 : N / 16;  // KIND 1: (gate, up) strip pairs; KIND 2: strips
   int64_t per = (G > 0) ? ((int64_t)T * K + G - 1) / G : 0;
-  if (extra_rows > per) per = extra_rows;
   if (per > (int64_t)T) per = T;
-  Plan p;
+  if (extra_rows > per) per = extra_rows;
+  Plan p{};
   p.tile = per > 128;
-  // a block covers 16*mt rows; leave head room over the mean so that a group rarely needs a
-  // second pass over its weights
-  p.mt = per <= 10 ? 1 : (per <= 21 ? 2 : 4);
-  p.nt = 1;
-  (void)kind; (void)N_strips_unit;
+  int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // tuning aid: 1 stream, 2 tile
+  if (force == 1) p.tile = false;
+  if (force == 2) p.tile = true;
+  if (p.tile && units % ((KIND == 1) ? 4 : 8) != 0) p.tile = false;
+  p.mt = per <= 10 ? 1 : 2;
+  p.S = 1;
+  if (KIND == 1) {
+    p.nt = 1; p.d = 4;
+  } else {
+    p.nt = 1; p.d = 4;
+  }
+  int s_env = 0;
+  if (const char* e = getenv(KIND == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2")) sscanf(e, "%d,%d,%d,%d", &p.mt, &p.nt, &p.d, &s_env);
+  if (Kdim % (64 * p.d) != 0) p.d = 4;
+  if (KIND == 1 && !p.tile && Kdim % 256 == 0 && units % (4 * p.nt) == 0) {
+    const int nchunks = Kdim / 256, dc = p.d / 4;
+    const int Gt = G + (extra_rows > 0 ? 1 : 0);
+    int64_t mb = (int64_t)Gt * ((per + 16 * p.mt - 1) / (16 * p.mt));
+    int64_t base = (int64_t)(units / (4 * p.nt)) * (mb > 0 ? mb : 1);
+    // measured on MI355X: extra k splits cost more in block start-up than they win back in the
+    // tail of the launch, so the default is one share; OMNI_MOE_G1="mt,nt,d,S" overrides
+    int want = 1;
+    (void)base;
+    if (s_env > 0) want = s_env;
+    int best = 1;
+    for (int sdiv = 1; sdiv <= nchunks; ++sdiv) {
+      if (nchunks % sdiv != 0 || (nchunks / sdiv) % dc != 0 || nchunks / sdiv < 2 * dc) continue;
+      if (sdiv <= want) best = sdiv;
+    }
+    p.S = best;
+  }
+  (void)M_cap;
   return p;
 }
 
@@ -470,7 +595,7 @@ void launch_stream(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) 
   const int BM = 16 * MT;
   const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
   int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
-  dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks), block(256);
+  dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks, (unsigned)a.S), block(256);
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }
 
@@ -484,47 +609,39 @@ void launch_tile(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
   hipLaunchKernelGGL((gemm_tile<KIND>), grid, block, 0, st, a);
 }
 
-int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : dflt;
-}
-
 template <int KIND>
-int dispatch_gemm(const GemmArgs& a, int64_t M_cap, hipStream_t st, const char* what) {
-  // units: KIND 1 -> (gate, up) strip pairs = I/16; KIND 2 -> strips = N/16
+int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, hipStream_t st, const char* what) {
   const int units = (KIND == 1) ? a.N / 32 : a.N / 16;
-  Plan p = choose_plan(KIND, a.T, a.K, a.G, a.extra_rows, units);
-  int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // 1 stream, 2 tile (tuning aid)
-  if (force == 1) p.tile = false;
-  if (force == 2) p.tile = true;
-  const int tile_units = (KIND == 1) ? 4 : 8;
-  if (p.tile && units % tile_units != 0) p.tile = false;
   if (p.tile) {
     launch_tile<KIND>(a, M_cap, units, st);
   } else {
-    if (units % 4 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: output channels %d not a multiple of %d", what, a.N, KIND == 1 ? 128 : 64);
-    int mt = env_int("OMNI_MOE_STREAM_MT", p.mt);
-    if constexpr (KIND == 1) {
-      if (mt <= 1) launch_stream<1, 1, 1, 8>(a, M_cap, units, st);
-      else if (mt == 2) launch_stream<1, 2, 1, 8>(a, M_cap, units, st);
-      else launch_stream<1, 4, 1, 4>(a, M_cap, units, st);
-    } else {
-      const bool nt4 = units % 16 == 0, nt2 = units % 8 == 0;
-      if (nt4) {
-        if (mt <= 1) launch_stream<2, 1, 4, 4>(a, M_cap, units, st);
-        else if (mt == 2) launch_stream<2, 2, 4, 4>(a, M_cap, units, st);
-        else launch_stream<2, 4, 4, 4>(a, M_cap, units, st);
-      } else if (nt2) {
-        if (mt <= 2) launch_stream<2, 2, 2, 4>(a, M_cap, units, st);
-        else launch_stream<2, 4, 2, 4>(a, M_cap, units, st);
-      } else {
-        if (mt <= 2) launch_stream<2, 2, 1, 4>(a, M_cap, units, st);
-        else launch_stream<2, 4, 1, 4>(a, M_cap, units, st);
-      }
-    }
+    const int mt = p.mt, nt = p.nt, d = p.d;
+    if (units % (4 * nt) != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: %d output strips not divisible by %d", what, units, 4 * nt);
+    if (a.Kdim % 256 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: reduction length %d must be a multiple of 256", what, a.Kdim);
+    bool ok = false;
+#define TRY(K_, MT_, NT_, D_)                                                  \
+  if (!ok && KIND == K_ && mt == MT_ && nt == NT_ && d == D_) {                \
+    if constexpr (KIND == K_) launch_stream<K_, MT_, NT_, D_>(a, M_cap, units, st); \
+    ok = true;                                                                 \
+  }
+    TRY(1, 1, 1, 4) TRY(1, 2, 1, 4) TRY(1, 4, 1, 4) TRY(1, 1, 1, 8) TRY(1, 2, 1, 8)
+    TRY(1, 1, 2, 4) TRY(1, 2, 2, 4) TRY(1, 4, 2, 4) TRY(1, 2, 2, 8)
+    TRY(2, 1, 1, 4) TRY(2, 2, 1, 4) TRY(2, 4, 1, 4) TRY(2, 1, 2, 4) TRY(2, 2, 2, 4) TRY(2, 4, 2, 4)
+    TRY(2, 1, 4, 4) TRY(2, 2, 4, 4) TRY(2, 2, 2, 8) TRY(2, 1, 2, 8) TRY(2, 2, 1, 8)
+#undef TRY
+    if (!ok) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: no stream kernel variant mt=%d nt=%d d=%d", what, mt, nt, d);
   }
   OMNI_CHECK_LAUNCH(what);
   return OMNI_OK;
+}
+
+size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
+  if (p.tile) {
+    size_t y = (size_t)M_cap * I * sizeof(float);
+    size_t rm = (((size_t)M_cap * sizeof(uint32_t)) + 255) / 256 * 256;
+    return y + rm + 256;
+  }
+  return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
 }
 
 int check_group_args(const char* what, const int32_t* offsets, int G, int H, int I, int64_t M_cap, int extra_rows,
@@ -539,11 +656,10 @@ int check_group_args(const char* what, const int32_t* offsets, int G, int H, int
 
 }  // namespace
 
-extern "C" size_t omni_moe_gemm1_workspace_bytes(int64_t M_cap, int I) {
-  if (M_cap < 0 || I <= 0) return 0;
-  size_t y = (size_t)M_cap * I * sizeof(float);
-  size_t rm = (((size_t)M_cap * sizeof(uint32_t)) + 255) / 256 * 256;
-  return y + rm + 256;
+extern "C" size_t omni_moe_gemm1_workspace_bytes(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I) {
+  if (M_cap < 0 || I <= 0 || H <= 0 || T < 0 || K <= 0 || G < 0) return 0;
+  Plan p = make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap);
+  return gemm1_ws_bytes(p, M_cap, I);
 }
 
 extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src,
@@ -557,25 +673,41 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   if (M_cap == 0) return OMNI_OK;
   if (!x_q || !x_scale || !h_q || !h_scale || (G > 0 && (!w13_packed || !w13_scale))) OMNI_FAIL(OMNI_E_INVALID, "gemm1: null pointer");
   if (T <= 0 || K <= 0) OMNI_FAIL(OMNI_E_INVALID, "gemm1: bad T=%d K=%d", T, K);
-  if (ws_bytes < omni_moe_gemm1_workspace_bytes(M_cap, I) || !workspace) OMNI_FAIL(OMNI_E_WORKSPACE, "gemm1: workspace %zu < %zu", ws_bytes, omni_moe_gemm1_workspace_bytes(M_cap, I));
+  Plan p = make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap);
+  const size_t need = gemm1_ws_bytes(p, M_cap, I);
+  if (ws_bytes < need || !workspace) OMNI_FAIL(OMNI_E_WORKSPACE, "gemm1: workspace %zu < %zu", ws_bytes, need);
   if (((uintptr_t)x_q % 16) || ((uintptr_t)w13_packed % 16) || ((uintptr_t)w13_extra % 16) || ((uintptr_t)workspace % 16) || ((uintptr_t)h_q % 4))
     OMNI_FAIL(OMNI_E_INVALID, "gemm1: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  float* y = (float*)workspace;
-  uint32_t* rowmax = (uint32_t*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
-  if (!(flags & OMNI_GEMM1_NO_PROLOGUE))
-    hipLaunchKernelGGL(zero_u32, dim3((unsigned)((M_cap + 255) / 256)), dim3(256), 0, st, rowmax, M_cap);
   GemmArgs a{};
   a.a_q = x_q; a.a_scale = x_scale; a.sorted_src = sorted_src; a.idx_mode = idx_mode; a.T = T; a.K = K;
   a.w = w13_packed; a.w_scale = w13_scale; a.w_extra = w13_extra; a.w_extra_scale = w13_extra_scale;
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = H; a.N = 2 * I; a.flags = flags;
-  a.y = y; a.rowmax = rowmax; a.acc_dbg = acc_dbg;
-  rc = dispatch_gemm<1>(a, M_cap, st, "gemm1");
+  a.acc_dbg = acc_dbg; a.S = p.S; a.M_cap = M_cap;
+  if (p.tile) {
+    // fused epilogue: y = silu(gate)*up to scratch, row maxima by atomic max, then a quantise pass
+    float* y = (float*)workspace;
+    uint32_t* rowmax = (uint32_t*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
+    a.y = y; a.rowmax = rowmax;
+    if (!(flags & OMNI_GEMM1_NO_PROLOGUE))
+      hipLaunchKernelGGL(zero_u32, dim3((unsigned)((M_cap + 255) / 256)), dim3(256), 0, st, rowmax, M_cap);
+    rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
+    if (rc) return rc;
+    if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
+    hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax, offsets, G,
+                       extra_rows, I, M_cap, h_q, h_scale);
+    OMNI_CHECK_LAUNCH("gemm1 quant");
+    return OMNI_OK;
+  }
+  // split-k stream kernel: raw int32 partial sums, then one row kernel does the whole epilogue
+  if (I > 256 * 16) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gemm1: intermediate size %d > 4096 in the small-batch path", I);
+  a.part = (int32_t*)workspace;
+  rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
   if (rc) return rc;
   if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
-  hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax, offsets, G,
-                     extra_rows, I, M_cap, h_q, h_scale);
-  OMNI_CHECK_LAUNCH("gemm1 quant");
+  if (I <= 256 * 8) hipLaunchKernelGGL(swiglu_quant_rows<8>, dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
+  else hipLaunchKernelGGL(swiglu_quant_rows<16>, dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
+  OMNI_CHECK_LAUNCH("gemm1 row epilogue");
   return OMNI_OK;
 }
 
@@ -595,8 +727,9 @@ extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, c
   a.T = (int)M_cap; a.K = 1;
   a.w = w2_packed; a.w_scale = w2_scale; a.w_extra = w2_extra; a.w_extra_scale = w2_extra_scale;
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = I; a.N = H; a.flags = 0;
-  a.rows_out = rows_out; a.out_dtype = out_dtype; a.acc_dbg = acc_dbg;
-  return dispatch_gemm<2>(a, M_cap, (hipStream_t)stream, "gemm2");
+  a.rows_out = rows_out; a.out_dtype = out_dtype; a.acc_dbg = acc_dbg; a.S = 1; a.M_cap = M_cap;
+  Plan p = make_plan<2>(a.T, a.K, G, extra_rows, I, H, M_cap);
+  return dispatch_gemm<2>(a, p, M_cap, (hipStream_t)stream, "gemm2");
 }
 
 extern "C" int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N, int8_t* packed,

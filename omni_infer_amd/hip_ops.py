@@ -224,7 +224,7 @@ def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_
     else:
         h_q, h_s = out
     acc = torch.zeros(M_cap, 2 * I, dtype=torch.int32, device=dev) if want_acc else None
-    ws_bytes = L.lib().omni_moe_gemm1_workspace_bytes(M_cap, I)
+    ws_bytes = L.lib().omni_moe_gemm1_workspace_bytes(T, K, G, extra_rows, M_cap, H, I)
     ws = workspace if workspace is not None else torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     ew, es = extra if extra is not None else (None, None)
     rc = L.lib().omni_moe_gemm1_swiglu_quant(
