@@ -18,8 +18,8 @@
 //                registers through a ring of D outstanding k-steps (each weight byte is used by
 //                exactly one wavefront, so LDS staging would only add traffic); A is small and
 //                shared by the four wavefronts of a block through LDS.
-//   gemm_tile    large row counts: 256 x 128 block tiles, A and B both staged through LDS with
-//                register prefetch of the next k-step, each wavefront a 128 x 64 sub-tile.
+//   gemm_pipe    large row counts: 256 x 128 block tiles, A and B both loaded straight into LDS
+//                through a three-stage ring, each wavefront a 128 x 64 sub-tile on 32x32x32 MFMAs.
 //
 // GEMM1 pairs gate channel n with up channel I + n in the same lane so SwiGLU needs no exchange.
 // Its epilogue writes y = silu(gate) * up in fp32 to a scratch matrix and folds max|y| of each
@@ -45,7 +45,8 @@ struct GemmArgs {
   int N;     // output channels of the GEMM: 2I (GEMM1) or H (GEMM2)
   int flags;
   float* y;            // GEMM1: [M_cap, I]
-  uint32_t* rowmax;    // GEMM1: [M_cap]
+  uint32_t* rowmax;    // unused by the kernels below (kept for layout stability)
+  float* rowmax_part;  // GEMM1 gemm_pipe: [M_cap, n_blocks] max|y| of every row within one channel block
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
   int32_t* acc_dbg;    // [M_cap, N], nullable
@@ -348,141 +349,270 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
 }
 
 // =====================================================================================
-// gemm_tile: block tile 256 rows x 128 channels (GEMM1: 64 gate + 64 up), k-step 64.
-//   four wavefronts as 2 (rows) x 2 (channels); a wavefront holds 8 x 4 accumulator tiles.
+// gemm_pipe: large row counts.  Block tile 256 rows x 128 channels (GEMM1: 64 gate + 64 up),
+// four wavefronts as 2 (rows) x 2 (channels), each a 128 x 64 sub-tile held as 4 x 2 accumulator
+// tiles of v_mfma_i32_32x32x32_i8 (a single wavefront issues the 32x32x32 form at nearly the
+// full MFMA rate, the 16x16x64 form at about half of it).
+//   Operands go from global memory straight into LDS (global_load_lds, 16 bytes per lane, no
+//   register staging) through a three-stage ring: while stage s is multiplied, stages s+1 and s+2
+//   are in flight.  A wavefront's load instruction moves one 1 KiB fragment of 16 rows (or 16
+//   channels) x 64 k, lane l -> bytes [16 l, 16 l + 16).  The 32x32x32 operand of lane l (row
+//   l%32, k-quarter 2*half + l/32 of the k-step) is then bytes
+//       fragment[(l%32)/16][ (l%16) + 16*(2*half + l/32) ]
+//   of two neighbouring fragments: groups of 16 lanes read 256 contiguous bytes.
+//   The stage buffers are separate __shared__ objects and the step function takes them as
+//   __restrict__ pointers: that is what lets the compiler see that the LDS reads of one stage do
+//   not alias the asynchronous writes into another, so it keeps the explicit
+//   "s_waitcnt vmcnt(loads of one stage)" and does not drain the ring before every LDS read.
 // =====================================================================================
-template <int KIND>
-__global__ __launch_bounds__(256, 2) void gemm_tile(GemmArgs a) {
-  constexpr int BM = 256, MTW = 8, NTW = 4;
-  __shared__ v4i lds_a[2][16 * WAVE];  // 16 fragments of 16 rows x 64 k
-  __shared__ v4i lds_b[2][8 * WAVE];   // 8 strips x 64 k
+#define OMNI_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+typedef int v16i __attribute__((ext_vector_type(16)));
 
-  const int lane = threadIdx.x & (WAVE - 1);
-  const int w = threadIdx.x / WAVE;
-  const int wm = w >> 1, wn = w & 1;
+template <int WN>
+struct PipeCtx {
+  static constexpr int NWAVES = 2 * WN;          // 2 wavefronts along the rows x WN along the channels
+  static constexpr int A_PER_WAVE = 16 / NWAVES; // A fragments (of 16) a wavefront loads per stage
+  static constexpr int LPS = A_PER_WAVE + 2;     // loads per stage per wavefront (2 B fragments each)
+  const int8_t* asrc[A_PER_WAVE];
+  const int8_t* bsrc[2];
+  int w, lane, wm, wn;
+  int a_off;     // v4i index of this lane's A operand inside the wavefront's first 32-row pair, half 0
+  int b_off[2];  // same for the two 32-channel tiles of the wavefront
+};
+
+template <int WN>
+__device__ __forceinline__ void pipe_load(const PipeCtx<WN>& c, int k, v4i* __restrict__ dst_a, v4i* __restrict__ dst_b) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
+  constexpr int AP = PipeCtx<WN>::A_PER_WAVE;
+#pragma unroll
+  for (int i = 0; i < AP; ++i)
+    __builtin_amdgcn_global_load_lds(c.asrc[i] + (size_t)k * 64, OMNI_LDS_PTR(dst_a + (AP * c.w + i) * WAVE), 16, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    __builtin_amdgcn_global_load_lds(c.bsrc[i] + (size_t)k * 1024, OMNI_LDS_PTR(dst_b + (2 * c.w + i) * WAVE), 16, 0, 0);
+#endif
+}
+
+template <int WN>
+__device__ __forceinline__ void pipe_step(const PipeCtx<WN>& c, int kload, v4i* __restrict__ dst_a,
+                                          v4i* __restrict__ dst_b, const v4i* __restrict__ src_a,
+                                          const v4i* __restrict__ src_b, v16i (&acc)[4][2]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  pipe_load<WN>(c, kload, dst_a, dst_b);
+  // operands of both halves: the second half is requested before the first half's MFMAs are issued,
+  // so its LDS latency hides behind them
+  v4i bf[2][2], af[2][4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) bf[0][t] = src_b[c.b_off[t]];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) af[0][mt] = src_a[c.a_off + mt * 2 * WAVE];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) bf[1][t] = src_b[c.b_off[t] + 32];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) af[1][mt] = src_a[c.a_off + mt * 2 * WAVE + 32];
+#pragma unroll
+  for (int half = 0; half < 2; ++half)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        acc[mt][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[half][mt], bf[half][t], acc[mt][t], 0, 0, 0);
+#endif
+}
+
+// wait until at most one stage of this wavefront's loads is still in flight, then meet the block
+template <int WN>
+__device__ __forceinline__ void pipe_sync() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int N = PipeCtx<WN>::LPS;
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));  // vmcnt(N), other counters untouched
+  __builtin_amdgcn_s_barrier();
+#endif
+}
+
+// 32x32 accumulator tile: lane l holds column l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
+__device__ __forceinline__ int tile32_row(int lane, int i) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }
+
+// WN = 2: 256 threads, tile 256 x 128, two blocks per CU.  WN = 4: 512 threads, tile 256 x 256, one block
+// per CU (a third fewer operand bytes through the vector memory path per MFMA).
+template <int KIND, int WN>
+__global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
+  constexpr int BM = 256;
+  constexpr int NBS = 4 * WN;             // B strips per stage
+  constexpr int GS = 2 * WN;              // KIND 1: gate strips per block
+  constexpr int AP = PipeCtx<WN>::A_PER_WAVE;
+  __shared__ v4i sa0[16 * WAVE], sa1[16 * WAVE], sa2[16 * WAVE];
+  __shared__ v4i sb0[NBS * WAVE], sb1[NBS * WAVE], sb2[NBS * WAVE];
+  __shared__ float row_scale[BM];     // activation scale of every row of the block
+  __shared__ float rmax_lds[WN][BM];  // GEMM1: max|y| per row, one column per wavefront column
+
+  PipeCtx<WN> c;
+  c.lane = threadIdx.x & (WAVE - 1);
+  c.w = threadIdx.x / WAVE;
+  c.wm = c.w / WN;
+  c.wn = c.w % WN;
+  const int lane = c.lane, w = c.w, wm = c.wm, wn = c.wn;
   RowBlock rb;
   if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, blockIdx.y, rb)) return;
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int nk64 = a.Kdim / 64;
   const int I = (KIND == 1) ? a.N / 2 : 0;
-
   const int8_t* wbase = (g < a.G) ? a.w + (size_t)g * a.Kdim * a.N : a.w_extra;
   const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
 
-  // the block's 8 strips: KIND 1: gate strips 4bx..4bx+3 then up strips; KIND 2: 8bx..8bx+7.
-  // block-level strip j (0..7); wavefront wn uses KIND 1: gate {2wn, 2wn+1}, up {4+2wn, 4+2wn+1};
-  // KIND 2: {4wn .. 4wn+3}.
+  // block-level strips j = 0..NBS-1: KIND 1: gate strips GS*bx.. then the matching up strips;
+  // KIND 2: strips NBS*bx...  A 32-channel tile is a pair of neighbouring strips.
   auto strip_of = [&](int j) -> int {
-    if constexpr (KIND == 1) return (j < 4) ? blockIdx.x * 4 + j : I / 16 + blockIdx.x * 4 + (j - 4);
-    else return blockIdx.x * 8 + j;
+    if constexpr (KIND == 1) return (j < GS) ? blockIdx.x * GS + j : I / 16 + blockIdx.x * GS + (j - GS);
+    else return blockIdx.x * NBS + j;
   };
-  // staging duties: A fragments 4w..4w+3 (rows 16*(4w+i) + lane%16), B strips 2w, 2w+1
-  const int8_t* arow[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int rr = (4 * w + i) * 16 + (lane & 15);
-    arow[i] = nullptr;
-    if (rr < nrows) arow[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (lane >> 4) * 16;
+  for (int i = 0; i < AP; ++i) {
+    int rr = (AP * w + i) * 16 + (lane & 15);
+    if (rr >= nrows) rr = 0;  // rows past the end alias the first row; their results are not stored
+    c.asrc[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (lane >> 4) * 16;
   }
-  const int8_t* bsrc[2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) bsrc[i] = wbase + (size_t)strip_of(2 * w + i) * nk64 * 1024 + lane * 16;
-
-  int bsel[NTW];  // block-level strip index of each of the wavefront's channel tiles
+  for (int i = 0; i < 2; ++i) c.bsrc[i] = wbase + (size_t)strip_of(2 * w + i) * nk64 * 1024 + lane * 16;
+  // per-row activation scales go to LDS once (read back in the epilogue)
+  for (int r = threadIdx.x; r < BM; r += 128 * WN) {
+    row_scale[r] = (r < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + r)] : 0.0f;
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) {
-    if constexpr (KIND == 1) bsel[t] = (t < 2) ? 2 * wn + t : 4 + 2 * wn + (t - 2);
-    else bsel[t] = 4 * wn + t;
+    for (int j = 0; j < WN; ++j) rmax_lds[j][r] = 0.0f;
   }
-
-  v4i acc[MTW][NTW];
-#pragma unroll
-  for (int mt = 0; mt < MTW; ++mt)
-#pragma unroll
-    for (int t = 0; t < NTW; ++t) acc[mt][t] = (v4i){0, 0, 0, 0};
-
-  v4i areg[4], breg[2];
-  auto fetch = [&](int ks) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      areg[i] = (v4i){0, 0, 0, 0};
-      if (arow[i]) areg[i] = *(const v4i*)(arow[i] + (size_t)ks * 64);
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) breg[i] = *(const v4i*)(bsrc[i] + (size_t)ks * 1024);
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) lds_a[buf][(4 * w + i) * WAVE + lane] = areg[i];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) lds_b[buf][(2 * w + i) * WAVE + lane] = breg[i];
-  };
-
-  fetch(0);
-  stash(0);
   __syncthreads();
-  const int mt_lim = min(MTW, (nrows - wm * 128 + 15) / 16);  // row tiles of this wavefront that hold rows
-  for (int ks = 0; ks < nk64; ++ks) {
-    const int buf = ks & 1;
-    if (ks + 1 < nk64) fetch(ks + 1);
-    v4i bf[NTW];
+  // operand addressing of the 32x32x32 form (see the header comment)
+  const int in_pair = ((lane & 31) >> 4) * WAVE + (lane & 15) + 16 * (lane >> 5);
+  c.a_off = (wm * 8) * WAVE + in_pair;
+  // wavefront column wn: KIND 1: gate tile = strips {2wn, 2wn+1}, up tile = strips {GS+2wn, GS+2wn+1};
+  //                      KIND 2: tiles = strips {4wn, 4wn+1} and {4wn+2, 4wn+3}
+  int tile_strip0[2];
+  if constexpr (KIND == 1) { tile_strip0[0] = 2 * wn; tile_strip0[1] = GS + 2 * wn; }
+  else { tile_strip0[0] = 4 * wn; tile_strip0[1] = 4 * wn + 2; }
 #pragma unroll
-    for (int t = 0; t < NTW; ++t) bf[t] = lds_b[buf][bsel[t] * WAVE + lane];
-#pragma unroll
-    for (int mt = 0; mt < MTW; ++mt) {
-      if (mt < mt_lim) {
-        v4i af = lds_a[buf][(wm * 8 + mt) * WAVE + lane];
-#pragma unroll
-        for (int t = 0; t < NTW; ++t) acc[mt][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, bf[t], acc[mt][t], 0, 0, 0);
-      }
-    }
-    if (ks + 1 < nk64) {
-      stash(buf ^ 1);
-      __syncthreads();
-    }
-  }
+  for (int t = 0; t < 2; ++t) c.b_off[t] = tile_strip0[t] * WAVE + in_pair;
 
-  const int col = lane & 15;
+  v16i acc[4][2];
 #pragma unroll
-  for (int mt = 0; mt < MTW; ++mt) {
-    if (mt < mt_lim) {
-      const int rbase = wm * 128 + mt * 16 + 4 * (lane >> 4);
-      float ts[4];
+  for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int rr = rbase + i;
-        ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
-      }
-      if constexpr (KIND == 1) {
-        float rmax[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          int n = (blockIdx.x * 4 + 2 * wn + t) * 16 + col;
-          epilogue_gemm1(a, g, wsc, I, n, row0, rbase, nrows, ts, acc[mt][t], acc[mt][2 + t], rmax);
-        }
-        flush_rowmax(a, row0, rbase, nrows, rmax);
-      } else {
+      for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
+
+  const int last = nk64 - 1;
+  pipe_load<WN>(c, 0, sa0, sb0);
+  pipe_load<WN>(c, min(1, last), sa1, sb1);
+  int ks = 0;
+  for (; ks + 3 <= nk64; ks += 3) {
+    pipe_sync<WN>();
+    pipe_step<WN>(c, min(ks + 2, last), sa2, sb2, sa0, sb0, acc);
+    pipe_sync<WN>();
+    pipe_step<WN>(c, min(ks + 3, last), sa0, sb0, sa1, sb1, acc);
+    pipe_sync<WN>();
+    pipe_step<WN>(c, min(ks + 4, last), sa1, sb1, sa2, sb2, acc);
+  }
+  if (ks < nk64) {  // one or two k-steps left; the ring is back at stage 0
+    pipe_sync<WN>();
+    pipe_step<WN>(c, last, sa2, sb2, sa0, sb0, acc);
+    if (ks + 1 < nk64) {
+      pipe_sync<WN>();
+      pipe_step<WN>(c, last, sa0, sb0, sa1, sb1, acc);
+    }
+  }
+  // no LDS traffic may still be in flight when the block's LDS is handed to the next block
+  __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));  // vmcnt(0)
+
+  // ---- epilogue, one 32-row tile at a time
+  const int c32 = lane & 31;
+  const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+  float wsc_g[2];
+  int ncol[2];
+  if constexpr (KIND == 1) {
+    ncol[0] = (blockIdx.x * GS + 2 * wn) * 16 + c32;
+    ncol[1] = I + ncol[0];
+  } else {
+    ncol[0] = (blockIdx.x * NBS + 4 * wn) * 16 + c32;
+    ncol[1] = ncol[0] + 32;
+  }
+  wsc_g[0] = wsc[ncol[0]];
+  wsc_g[1] = wsc[ncol[1]];
 #pragma unroll
-        for (int t = 0; t < NTW; ++t) {
-          int n = (blockIdx.x * 8 + 4 * wn + t) * 16 + col;
-          epilogue_gemm2(a, wsc, n, row0, rbase, nrows, ts, acc[mt][t]);
+  for (int mt = 0; mt < 4; ++mt) {
+    const int tile_r0 = wm * 128 + mt * 32;
+    if (tile_r0 < nrows) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int rr = tile_r0 + tile32_row(lane, i);
+        const bool ok = rr < nrows;
+        const size_t m = (size_t)(row0 + rr);
+        const float ts = row_scale[rr];
+        if constexpr (KIND == 1) {
+          float yv = 0.0f;
+          if (ok) {
+            float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
+            float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
+            if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+            yv = silu_spec(dg) * du;
+            if (bf) yv = round_bf16(yv);
+            a.y[m * I + ncol[0]] = yv;
+            if (a.acc_dbg) {
+              a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
+              a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
+            }
+          }
+          // max |y| over the 32 lanes that hold this row
+          float mx = fabsf(yv);
+          mx = fmaxf(mx, xchg_f<1>(mx));
+          mx = fmaxf(mx, xchg_f<2>(mx));
+          mx = fmaxf(mx, xchg_f<4>(mx));
+          mx = fmaxf(mx, xchg_f<8>(mx));
+          mx = fmaxf(mx, xchg_f<16>(mx));
+          if (c32 == 0) rmax_lds[wn][rr] = mx;
+        } else {
+          if (ok) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              float o = ((float)acc[mt][t][i] * wsc_g[t]) * ts;
+              if (a.out_dtype == OMNI_DT_F32) ((float*)a.rows_out)[m * (size_t)a.N + ncol[t]] = o;
+              else ((uint16_t*)a.rows_out)[m * (size_t)a.N + ncol[t]] = f32_to_bf16(o);
+              if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + ncol[t]] = acc[mt][t][i];
+            }
+          }
         }
       }
     }
   }
+  if constexpr (KIND == 1) {
+    // one word per (row, channel block): the quantise pass takes the maximum over the blocks;
+    // no atomics, nothing to clear beforehand
+    __syncthreads();
+    for (int r = threadIdx.x; r < nrows; r += 128 * WN) {
+      float mx = rmax_lds[0][r];
+#pragma unroll
+      for (int j = 1; j < WN; ++j) mx = fmaxf(mx, rmax_lds[j][r]);
+      a.rowmax_part[(size_t)(row0 + r) * gridDim.x + blockIdx.x] = mx;
+    }
+  }
+#endif
 }
 
 // =====================================================================================
 // row quantisation of y with the row maximum already known (one wavefront per row)
 // =====================================================================================
-__global__ __launch_bounds__(256) void quant_known_max(const float* __restrict__ y, const uint32_t* __restrict__ rowmax,
-                                                       const int32_t* __restrict__ offsets, int G, int extra_rows, int I,
-                                                       int64_t M_cap, int8_t* __restrict__ hq, float* __restrict__ hs) {
+__global__ __launch_bounds__(256) void quant_known_max(const float* __restrict__ y, const float* __restrict__ rowmax_part,
+                                                       int nparts, const int32_t* __restrict__ offsets, int G,
+                                                       int extra_rows, int I, int64_t M_cap, int8_t* __restrict__ hq,
+                                                       float* __restrict__ hs) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int64_t m = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
   const int64_t total = (int64_t)offsets[G] + extra_rows;
   if (m >= total || m >= M_cap) return;
-  const float s = __uint_as_float(rowmax[m]) / 127.0f;
+  float mx = 0.0f;
+  for (int p = lane; p < nparts; p += WAVE) mx = fmaxf(mx, rowmax_part[m * nparts + p]);
+  mx = wave_allmax_f(mx);
+  const float s = mx / 127.0f;
   if (lane == 0) hs[m] = s;
   const float* yr = y + m * I;
   int8_t* qr = hq + m * I;
@@ -599,14 +729,25 @@ void launch_stream(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) 
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }
 
+// number of channel blocks of the large-tile GEMM1 (also the number of row-maximum words per row)
+int tile_wn(int kind, int units) {
+  const int wide = (kind == 1) ? 8 : 16;  // units per 256-channel block
+  const int want = env_int("OMNI_MOE_TILE_WN", 4);
+  return (want == 4 && units % wide == 0) ? 4 : 2;
+}
+
 template <int KIND>
 void launch_tile(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
   const int BM = 256;
   const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
   int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
-  const int per_block = (KIND == 1) ? 4 : 8;
-  dim3 grid((unsigned)(units / per_block), (unsigned)mblocks), block(256);
-  hipLaunchKernelGGL((gemm_tile<KIND>), grid, block, 0, st, a);
+  if (tile_wn(KIND, units) == 4) {
+    dim3 grid((unsigned)(units / ((KIND == 1) ? 8 : 16)), (unsigned)mblocks), block(512);
+    hipLaunchKernelGGL((gemm_pipe<KIND, 4>), grid, block, 0, st, a);
+  } else {
+    dim3 grid((unsigned)(units / ((KIND == 1) ? 4 : 8)), (unsigned)mblocks), block(256);
+    hipLaunchKernelGGL((gemm_pipe<KIND, 2>), grid, block, 0, st, a);
+  }
 }
 
 template <int KIND>
@@ -638,7 +779,7 @@ int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, hipStream_t s
 size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
   if (p.tile) {
     size_t y = (size_t)M_cap * I * sizeof(float);
-    size_t rm = (((size_t)M_cap * sizeof(uint32_t)) + 255) / 256 * 256;
+    size_t rm = (((size_t)M_cap * (I / 64) * sizeof(float)) + 255) / 256 * 256;  // one word per row and 64-channel block
     return y + rm + 256;
   }
   return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
@@ -685,17 +826,16 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = H; a.N = 2 * I; a.flags = flags;
   a.acc_dbg = acc_dbg; a.S = p.S; a.M_cap = M_cap;
   if (p.tile) {
-    // fused epilogue: y = silu(gate)*up to scratch, row maxima by atomic max, then a quantise pass
+    // fused epilogue: y = silu(gate)*up to scratch with per-block row maxima, then a quantise pass
     float* y = (float*)workspace;
-    uint32_t* rowmax = (uint32_t*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
-    a.y = y; a.rowmax = rowmax;
-    if (!(flags & OMNI_GEMM1_NO_PROLOGUE))
-      hipLaunchKernelGGL(zero_u32, dim3((unsigned)((M_cap + 255) / 256)), dim3(256), 0, st, rowmax, M_cap);
+    float* rowmax_part = (float*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
+    a.y = y; a.rowmax_part = rowmax_part;
     rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
-    hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax, offsets, G,
-                       extra_rows, I, M_cap, h_q, h_scale);
+    const int nparts = (tile_wn(1, I / 16) == 4) ? I / 128 : I / 64;  // = grid.x of the GEMM launch
+    hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax_part, nparts,
+                       offsets, G, extra_rows, I, M_cap, h_q, h_scale);
     OMNI_CHECK_LAUNCH("gemm1 quant");
     return OMNI_OK;
   }
