@@ -152,7 +152,13 @@ struct LayerWs {
   size_t x_q, x_s, sorted_src, src_to_dst, counts, offsets, perm_ws, h_q, h_s, g1_ws, rows, total;
   size_t perm_bytes, g1_bytes;
   int64_t M_cap;
+  int rows_dtype;
 };
+// The expert rows between GEMM2 and the combine are kept in fp32 (the numerics of the fused
+// GEMM2+finalize operator) while that buffer stays within the 256 MiB last-level cache; beyond it
+// they are rounded to bf16 (the numerics of the separate GEMM2 and finalize operators), which
+// halves the largest intermediate of a prefill-sized call.
+constexpr size_t ROWS_F32_LIMIT = (size_t)256 << 20;
 LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
   LayerWs L{};
   L.M_cap = (int64_t)T * K + (with_shared ? T : 0);
@@ -170,7 +176,8 @@ LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
   L.h_s = take((size_t)L.M_cap * 4);
   L.g1_bytes = omni_moe_gemm1_workspace_bytes(T, K, G, with_shared ? T : 0, L.M_cap, H, I);
   L.g1_ws = take(L.g1_bytes);
-  L.rows = take((size_t)L.M_cap * H * 4);
+  L.rows_dtype = ((size_t)L.M_cap * H * 4 <= ROWS_F32_LIMIT) ? OMNI_DT_F32 : OMNI_DT_BF16;
+  L.rows = take((size_t)L.M_cap * H * (L.rows_dtype == OMNI_DT_F32 ? 4 : 2));
   L.total = o;
   return L;
 }
@@ -219,9 +226,9 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
                                    (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, stream);
   if (rc) return rc;
   rc = omni_moe_gemm2_dequant((const int8_t*)(ws + L.h_q), (const float*)(ws + L.h_s), w2_packed, w2_scale, sh2_packed,
-                              sh2_scale, extra, offsets, G, H, I, L.M_cap, OMNI_DT_F32, ws + L.rows, nullptr, stream);
+                              sh2_scale, extra, offsets, G, H, I, L.M_cap, L.rows_dtype, ws + L.rows, nullptr, stream);
   if (rc) return rc;
-  return omni_moe_combine(ws + L.rows, OMNI_DT_F32, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
+  return omni_moe_combine(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
                           nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,
                           stream);
 }

@@ -133,8 +133,14 @@ __device__ __forceinline__ void flush_rowmax(const GemmArgs& a, int row0, int rb
 // the loop is split into a part that refills the ring and a drain part, so the compiler can
 // count outstanding loads exactly and never waits for more than the oldest k-step.
 // =====================================================================================
+// Occupancy asked of the compiler: the small variants are held to 5 wavefronts per SIMD (96
+// registers) so that a decode-sized launch (about 34 row blocks x 32 channel blocks) is resident
+// all at once: a second, nearly empty round of blocks would stream at a fraction of the bandwidth.
 template <int KIND, int MT, int NT, int D>
-__global__ __launch_bounds__(256) void gemm_stream(GemmArgs a) {
+constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1; }
+
+template <int KIND, int MT, int NT, int D>
+__global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void gemm_stream(GemmArgs a) {
   constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
   constexpr int BM = 16 * MT;
   constexpr int DC = D / 4;                       // chunks (4 k-steps) of B in flight
