@@ -60,30 +60,34 @@ __device__ __forceinline__ void load4(const void* base, size_t row, int H, int c
 
 template <int DT>
 __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
-  __shared__ int s_slot[KMAX];
+  __shared__ int s_slot[KMAX], s_raw[KMAX];
   __shared__ float s_w[KMAX];
-  __shared__ int s_cnt;
   const int n = blockIdx.x;
-  if (threadIdx.x == 0) {
-    int cnt = 0;
-    for (int k = 0; k < a.K; ++k) {
-      int idx = (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? n * a.K + k : k * a.T + n;
-      int slot = a.src_to_dst[idx];
-      if (slot < 0) continue;
-      float wv = a.topk_w[(size_t)n * a.K + k];
-      int pos = cnt;
-      if (a.order == OMNI_ORDER_SLOT) {  // insertion by slot; k order otherwise
-        while (pos > 0 && s_slot[pos - 1] > slot) {
-          s_slot[pos] = s_slot[pos - 1];
-          s_w[pos] = s_w[pos - 1];
-          --pos;
-        }
-      }
+  // thread k fetches assignment k; its place in the list is the number of kept assignments that
+  // come before it (lower slot, or lower k, as the order asks)
+  int slot = -1;
+  float wv = 0.0f;
+  if (threadIdx.x < a.K) {
+    const int k = threadIdx.x;
+    const int idx = (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? n * a.K + k : k * a.T + n;
+    slot = a.src_to_dst[idx];
+    wv = a.topk_w[(size_t)n * a.K + k];
+    s_raw[k] = slot;
+  }
+  __syncthreads();
+  int cnt = 0;
+  {
+    int pos = 0;
+    for (int j = 0; j < a.K; ++j) {
+      const int sj = s_raw[j];
+      if (sj < 0) continue;
+      ++cnt;
+      if (a.order == OMNI_ORDER_SLOT ? (sj < slot) : (j < (int)threadIdx.x)) ++pos;
+    }
+    if (threadIdx.x < a.K && slot >= 0) {
       s_slot[pos] = slot;
       s_w[pos] = wv;
-      ++cnt;
     }
-    s_cnt = cnt;
   }
   __syncthreads();
   const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
@@ -91,7 +95,6 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
   const int ncol = min(4, a.H - c);
   float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if (a.init) load4<OMNI_DT_BF16>(a.init, (size_t)n, a.H, c, ncol, acc);
-  const int cnt = s_cnt;
   for (int j = 0; j < cnt; ++j) {
     float v[4];
     load4<DT>(a.rows, (size_t)s_slot[j], a.H, c, ncol, v);

@@ -67,6 +67,16 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return (uint16_t)(u >> 16);
 }
+// two values at once with the hardware conversion (round to nearest even): low half = a, high half = b
+typedef float omni_f2 __attribute__((ext_vector_type(2)));
+typedef __bf16 omni_bf2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float a, float b) {
+  omni_f2 v = {a, b};
+  omni_bf2 r = __builtin_convertvector(v, omni_bf2);
+  uint32_t u;
+  __builtin_memcpy(&u, &r, 4);
+  return u;
+}
 __device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 __device__ __forceinline__ float f16_to_f32(uint16_t h) {
   _Float16 v;
@@ -123,6 +133,20 @@ __device__ __forceinline__ uint64_t wave_allmax_u64(uint64_t v) {
   o = xchg_u64<16>(v); v = o > v ? o : v;
   o = xchg_u64<32>(v); v = o > v ? o : v;
   return v;
+}
+// wave-wide max of unsigned keys: four DPP steps inside each row of 16 lanes, then the four row
+// results are read through scalar registers (no LDS-crossbar permutes)
+__device__ __forceinline__ uint32_t wave_allmax_u32(uint32_t v) {
+  uint32_t o;
+  o = (uint32_t)xchg_i<1>((int)v); v = o > v ? o : v;
+  o = (uint32_t)xchg_i<2>((int)v); v = o > v ? o : v;
+  o = (uint32_t)xchg_i<4>((int)v); v = o > v ? o : v;
+  o = (uint32_t)xchg_i<8>((int)v); v = o > v ? o : v;
+  uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+  uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+  r0 = r0 > r1 ? r0 : r1;
+  r2 = r2 > r3 ? r2 : r3;
+  return r0 > r2 ? r0 : r2;
 }
 // max over the 16 lanes of a DPP row
 __device__ __forceinline__ float row16_allmax_f(float v) {

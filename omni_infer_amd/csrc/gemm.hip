@@ -45,8 +45,6 @@ struct GemmArgs {
   int N;     // output channels of the GEMM: 2I (GEMM1) or H (GEMM2)
   int flags;
   float* y;            // GEMM1: [M_cap, I]
-  uint32_t* rowmax;    // unused by the kernels below (kept for layout stability)
-  float* rowmax_part;  // GEMM1 gemm_pipe: [M_cap, n_blocks] max|y| of every row within one channel block
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
   int32_t* acc_dbg;    // [M_cap, N], nullable
@@ -68,32 +66,6 @@ __device__ __forceinline__ int source_row(const GemmArgs& a, int g, int r) {
   }
 }
 
-// Epilogue of one 16x16 gate/up tile pair of GEMM1.  rows: row0 + rbase + i (i < 4) for this lane.
-__device__ __forceinline__ void epilogue_gemm1(const GemmArgs& a, int g, const float* __restrict__ wsc, int I, int n,
-                                               int row0, int rbase, int nrows, const float* ts, v4i accg, v4i accu,
-                                               float* rmax) {
-  const float wg = wsc[n], wu = wsc[I + n];
-  const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int rr = rbase + i;
-    if (rr < nrows) {
-      float dg = ((float)accg[i] * wg) * ts[i];
-      float du = ((float)accu[i] * wu) * ts[i];
-      if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
-      float yv = silu_spec(dg) * du;
-      if (bf) yv = round_bf16(yv);
-      size_t m = (size_t)(row0 + rr);
-      a.y[m * I + n] = yv;
-      rmax[i] = fmaxf(rmax[i], fabsf(yv));
-      if (a.acc_dbg) {
-        a.acc_dbg[m * (size_t)a.N + n] = accg[i];
-        a.acc_dbg[m * (size_t)a.N + I + n] = accu[i];
-      }
-    }
-  }
-}
-
 __device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float* __restrict__ wsc, int n, int row0,
                                                int rbase, int nrows, const float* ts, v4i acc) {
   const float ws = wsc[n];
@@ -107,17 +79,6 @@ __device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float* _
       else ((uint16_t*)a.rows_out)[m * (size_t)a.N + n] = f32_to_bf16(o);
       if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + n] = acc[i];
     }
-  }
-}
-
-// fold the lane's row maxima over the 16 lanes that hold the same rows, then one atomic per row
-__device__ __forceinline__ void flush_rowmax(const GemmArgs& a, int row0, int rbase, int nrows, float* rmax) {
-  const int lane = threadIdx.x & (WAVE - 1);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float m = row16_allmax_f(rmax[i]);
-    int rr = rbase + i;
-    if ((lane & 15) == 0 && rr < nrows) atomicMax(&a.rowmax[row0 + rr], __float_as_uint(m));
   }
 }
 
@@ -294,20 +255,17 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
   __shared__ float red[4];
   __shared__ int s_group;
   const int64_t m = blockIdx.x;
-  const int64_t total = (int64_t)a.offsets[a.G] + a.extra_rows;
-  if (m >= total) return;
-  if (threadIdx.x == 0) {
-    int lo = 0, hi = a.G;  // group g with offsets[g] <= m < offsets[g+1]; rows past offsets[G]: extra group
-    if (m >= a.offsets[a.G]) lo = a.G;
-    else {
-      while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (a.offsets[mid] <= m) lo = mid; else hi = mid;
-      }
-    }
-    s_group = lo;
+  // group g with offsets[g] <= m < offsets[g+1] (rows from offsets[G] on: the extra group); one
+  // thread per group looks, so the lookup costs one round trip to memory
+  if (threadIdx.x == 0) s_group = -1;
+  __syncthreads();
+  for (int g = threadIdx.x; g <= a.G; g += 256) {
+    const int64_t lo = a.offsets[g];
+    const int64_t hi = (g < a.G) ? (int64_t)a.offsets[g + 1] : lo + a.extra_rows;
+    if (m >= lo && m < hi) s_group = g;
   }
   __syncthreads();
+  if (s_group < 0) return;  // past the last row
   const int g = s_group;
   const int I = a.N / 2;
   const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
@@ -451,7 +409,6 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   __shared__ v4i sa0[16 * WAVE], sa1[16 * WAVE], sa2[16 * WAVE];
   __shared__ v4i sb0[NBS * WAVE], sb1[NBS * WAVE], sb2[NBS * WAVE];
   __shared__ float row_scale[BM];     // activation scale of every row of the block
-  __shared__ float rmax_lds[WN][BM];  // GEMM1: max|y| per row, one column per wavefront column
 
   PipeCtx<WN> c;
   c.lane = threadIdx.x & (WAVE - 1);
@@ -484,8 +441,6 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // per-row activation scales go to LDS once (read back in the epilogue)
   for (int r = threadIdx.x; r < BM; r += 128 * WN) {
     row_scale[r] = (r < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + r)] : 0.0f;
-#pragma unroll
-    for (int j = 0; j < WN; ++j) rmax_lds[j][r] = 0.0f;
   }
   __syncthreads();
   // operand addressing of the 32x32x32 form (see the header comment)
@@ -532,6 +487,12 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 
   // ---- epilogue, one 32-row tile at a time
   const int c32 = lane & 31;
+  // bf16 rows of GEMM2 are transposed through LDS (the stage buffers are free now): a private
+  // 32 x 64 piece per wavefront, rows padded to 144 bytes; three wavefronts share a stage buffer
+  constexpr int OUT_PITCH = 72;  // uint16 elements
+  const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
+  uint16_t* stage16 = (uint16_t*)(w < 3 ? sa0 : (w < 6 ? sa1 : sa2)) + (w % 3) * (32 * OUT_PITCH);
+  if (bf16_out) __syncthreads();  // every wavefront is done reading the last stage
   const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
   float wsc_g[2];
   int ncol[2];
@@ -555,87 +516,119 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
         const size_t m = (size_t)(row0 + rr);
         const float ts = row_scale[rr];
         if constexpr (KIND == 1) {
-          float yv = 0.0f;
           if (ok) {
             float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
             float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
             if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
-            yv = silu_spec(dg) * du;
+            float yv = silu_spec(dg) * du;
             if (bf) yv = round_bf16(yv);
-            a.y[m * I + ncol[0]] = yv;
+            __builtin_nontemporal_store(yv, &a.y[m * I + ncol[0]]);  // read once, by the row quantiser
             if (a.acc_dbg) {
               a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
               a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
             }
           }
-          // max |y| over the 32 lanes that hold this row
-          float mx = fabsf(yv);
-          mx = fmaxf(mx, xchg_f<1>(mx));
-          mx = fmaxf(mx, xchg_f<2>(mx));
-          mx = fmaxf(mx, xchg_f<4>(mx));
-          mx = fmaxf(mx, xchg_f<8>(mx));
-          mx = fmaxf(mx, xchg_f<16>(mx));
-          if (c32 == 0) rmax_lds[wn][rr] = mx;
         } else {
-          if (ok) {
+          if (bf16_out) {
+            // through LDS: the tile's 64 channels of a row become one 128-byte line
+            const float o0 = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
+            const float o1 = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
+            const uint32_t pk = f32x2_to_bf16x2(o0, o1);
+            stage16[tile32_row(lane, i) * OUT_PITCH + c32] = (uint16_t)(pk & 0xffffu);
+            stage16[tile32_row(lane, i) * OUT_PITCH + 32 + c32] = (uint16_t)(pk >> 16);
+            if (ok && a.acc_dbg) {
+              a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
+              a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
+            }
+          } else if (ok) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
               float o = ((float)acc[mt][t][i] * wsc_g[t]) * ts;
-              if (a.out_dtype == OMNI_DT_F32) ((float*)a.rows_out)[m * (size_t)a.N + ncol[t]] = o;
-              else ((uint16_t*)a.rows_out)[m * (size_t)a.N + ncol[t]] = f32_to_bf16(o);
+              __builtin_nontemporal_store(o, &((float*)a.rows_out)[m * (size_t)a.N + ncol[t]]);
               if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + ncol[t]] = acc[mt][t][i];
             }
           }
         }
       }
-    }
-  }
-  if constexpr (KIND == 1) {
-    // one word per (row, channel block): the quantise pass takes the maximum over the blocks;
-    // no atomics, nothing to clear beforehand
-    __syncthreads();
-    for (int r = threadIdx.x; r < nrows; r += 128 * WN) {
-      float mx = rmax_lds[0][r];
+      if constexpr (KIND == 2) {
+        if (bf16_out) {
+          // the wavefront wrote its 32 x 64 piece; now 8 lanes per row store 16 bytes each
+          __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int j = 1; j < WN; ++j) mx = fmaxf(mx, rmax_lds[j][r]);
-      a.rowmax_part[(size_t)(row0 + r) * gridDim.x + blockIdx.x] = mx;
+          for (int j = 0; j < 4; ++j) {
+            const int r = j * 8 + (lane >> 3);
+            const int rr = tile_r0 + r;
+            v4i v = *(const v4i*)(stage16 + r * OUT_PITCH + (lane & 7) * 8);
+            if (rr < nrows)  // read once, by the combine
+              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
     }
   }
 #endif
 }
 
 // =====================================================================================
-// row quantisation of y with the row maximum already known (one wavefront per row)
+// row quantisation of y = silu(gate) * up (fp32, written by gemm_pipe): one wavefront per row keeps
+// up to 256*NV values in registers between the max|y| reduction and the rounding, so the row is read
+// once; NV == 0 reads it twice
 // =====================================================================================
-__global__ __launch_bounds__(256) void quant_known_max(const float* __restrict__ y, const float* __restrict__ rowmax_part,
-                                                       int nparts, const int32_t* __restrict__ offsets, int G,
-                                                       int extra_rows, int I, int64_t M_cap, int8_t* __restrict__ hq,
-                                                       float* __restrict__ hs) {
+template <int NV>
+__global__ __launch_bounds__(256) void quant_rows_y(const float* __restrict__ y, const int32_t* __restrict__ offsets,
+                                                    int G, int extra_rows, int I, int64_t M_cap,
+                                                    int8_t* __restrict__ hq, float* __restrict__ hs) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int64_t m = (int64_t)blockIdx.x * 4 + threadIdx.x / WAVE;
   const int64_t total = (int64_t)offsets[G] + extra_rows;
   if (m >= total || m >= M_cap) return;
-  float mx = 0.0f;
-  for (int p = lane; p < nparts; p += WAVE) mx = fmaxf(mx, rowmax_part[m * nparts + p]);
-  mx = wave_allmax_f(mx);
-  const float s = mx / 127.0f;
-  if (lane == 0) hs[m] = s;
   const float* yr = y + m * I;
   int8_t* qr = hq + m * I;
-  for (int c = lane * 4; c < I; c += WAVE * 4) {
-    v4f v = *(const v4f*)(yr + c);
-    uint32_t o = 0;
-    if (s > 0.0f) {
+  float mx = 0.0f;
+  if constexpr (NV > 0) {
+    v4f v[NV];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o |= ((uint32_t)(quant_i8(v[j], s) & 0xff)) << (8 * j);
+    for (int i = 0; i < NV; ++i) {
+      const int c = (i * WAVE + lane) * 4;
+      v[i] = (c < I) ? __builtin_nontemporal_load((const v4f*)(yr + c)) : (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(v[i][j]));
     }
-    *(uint32_t*)(qr + c) = o;
+    mx = wave_allmax_f(mx);
+    const float s = mx / 127.0f;
+    if (lane == 0) hs[m] = s;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = (i * WAVE + lane) * 4;
+      if (c < I) {
+        uint32_t o = 0;
+        if (s > 0.0f) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o |= ((uint32_t)(quant_i8(v[i][j], s) & 0xff)) << (8 * j);
+        }
+        *(uint32_t*)(qr + c) = o;
+      }
+    }
+  } else {
+    for (int c = lane * 4; c < I; c += WAVE * 4) {
+      v4f v = *(const v4f*)(yr + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(v[j]));
+    }
+    mx = wave_allmax_f(mx);
+    const float s = mx / 127.0f;
+    if (lane == 0) hs[m] = s;
+    for (int c = lane * 4; c < I; c += WAVE * 4) {
+      v4f v = *(const v4f*)(yr + c);
+      uint32_t o = 0;
+      if (s > 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o |= ((uint32_t)(quant_i8(v[j], s) & 0xff)) << (8 * j);
+      }
+      *(uint32_t*)(qr + c) = o;
+    }
   }
-}
-
-__global__ __launch_bounds__(256) void zero_u32(uint32_t* p, int64_t n) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = 0u;
 }
 
 // ---------------------------------------------------------------- weight packing
@@ -673,6 +666,7 @@ struct Plan {
   bool tile;
   int mt, nt, d;  // stream kernel parameters
   int S;          // k splits (GEMM1 stream kernel only)
+  int64_t per;    // expected rows of a busy group
 };
 
 int env_int(const char* name, int dflt) {
@@ -690,6 +684,7 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
   if (per > (int64_t)T) per = T;
   if (extra_rows > per) per = extra_rows;
   Plan p{};
+  p.per = per;
   p.tile = per > 128;
   int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // tuning aid: 1 stream, 2 tile
   if (force == 1) p.tile = false;
@@ -784,9 +779,7 @@ int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, hipStream_t s
 
 size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
   if (p.tile) {
-    size_t y = (size_t)M_cap * I * sizeof(float);
-    size_t rm = (((size_t)M_cap * (I / 64) * sizeof(float)) + 255) / 256 * 256;  // one word per row and 64-channel block
-    return y + rm + 256;
+    return (size_t)M_cap * I * sizeof(float) + 256;  // y = silu(gate) * up before the row quantiser
   }
   return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
 }
@@ -832,16 +825,17 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = H; a.N = 2 * I; a.flags = flags;
   a.acc_dbg = acc_dbg; a.S = p.S; a.M_cap = M_cap;
   if (p.tile) {
-    // fused epilogue: y = silu(gate)*up to scratch with per-block row maxima, then a quantise pass
+    // fused epilogue: y = silu(gate)*up to scratch, then the row quantiser
     float* y = (float*)workspace;
-    float* rowmax_part = (float*)((char*)workspace + (size_t)M_cap * I * sizeof(float));
-    a.y = y; a.rowmax_part = rowmax_part;
+    a.y = y;
     rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
-    const int nparts = (tile_wn(1, I / 16) == 4) ? I / 128 : I / 64;  // = grid.x of the GEMM launch
-    hipLaunchKernelGGL(quant_known_max, dim3((unsigned)((M_cap + 3) / 4)), dim3(256), 0, st, y, rowmax_part, nparts,
-                       offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+    dim3 qgrid((unsigned)((M_cap + 3) / 4)), qblock(256);
+    if (I <= 256 * 4) hipLaunchKernelGGL(quant_rows_y<4>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+    else if (I <= 256 * 8) hipLaunchKernelGGL(quant_rows_y<8>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+    else if (I <= 256 * 16) hipLaunchKernelGGL(quant_rows_y<16>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+    else hipLaunchKernelGGL(quant_rows_y<0>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
     OMNI_CHECK_LAUNCH("gemm1 quant");
     return OMNI_OK;
   }

@@ -67,17 +67,6 @@ __global__ __launch_bounds__(256) void route_kernel(RouteArgs a) {
 #pragma unroll
     for (int j = 0; j < V; ++j) ge[j] = (lane * V + j) / gsz;
     float my_gs = NEG_INF;  // lane g keeps the score of group g
-    for (int g = 0; g < a.n_group; ++g) {
-      float a1 = NEG_INF, a2 = NEG_INF;
-#pragma unroll
-      for (int j = 0; j < V; ++j) {
-        if (in[j] && ge[j] == g) {
-          float v = c[j];
-          if (v > a1) { a2 = a1; a1 = v; }
-          else if (v > a2) { a2 = v; }
-        }
-      }
-      // butterfly merge of (largest, second largest)
 #define MERGE2(S)                                         \
   {                                                       \
     float b1 = xchg_f<S>(a1), b2 = xchg_f<S>(a2);         \
@@ -85,54 +74,87 @@ __global__ __launch_bounds__(256) void route_kernel(RouteArgs a) {
     float n2 = fmaxf(fminf(a1, b1), fmaxf(a2, b2));       \
     a1 = n1; a2 = n2;                                     \
   }
-      MERGE2(1) MERGE2(2) MERGE2(4) MERGE2(8) MERGE2(16) MERGE2(32)
-#undef MERGE2
+    const int L = gsz / V;  // lanes per group when a group is a whole power-of-two run of lanes
+    if (gsz % V == 0 && (L & (L - 1)) == 0 && a.E == WAVE * V) {
+      // every group at once: (largest, second largest) merged inside each run of L lanes
+      float a1 = NEG_INF, a2 = NEG_INF;
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        float v = c[j];
+        if (v > a1) { a2 = a1; a1 = v; }
+        else if (v > a2) { a2 = v; }
+      }
+      if (L > 1) MERGE2(1)
+      if (L > 2) MERGE2(2)
+      if (L > 4) MERGE2(4)
+      if (L > 8) MERGE2(8)
+      if (L > 16) MERGE2(16)
+      if (L > 32) MERGE2(32)
       float gs = (a.group_mode == OMNI_GROUP_TOP2SUM) ? a1 + a2 : a1;
-      if (lane == g) my_gs = gs;
+      my_gs = __shfl(gs, (lane < a.n_group) ? lane * L : 0, WAVE);
+    } else {
+      for (int g = 0; g < a.n_group; ++g) {
+        float a1 = NEG_INF, a2 = NEG_INF;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          if (in[j] && ge[j] == g) {
+            float v = c[j];
+            if (v > a1) { a2 = a1; a1 = v; }
+            else if (v > a2) { a2 = v; }
+          }
+        }
+        MERGE2(1) MERGE2(2) MERGE2(4) MERGE2(8) MERGE2(16) MERGE2(32)
+        float gs = (a.group_mode == OMNI_GROUP_TOP2SUM) ? a1 + a2 : a1;
+        if (lane == g) my_gs = gs;
+      }
     }
-    uint64_t kept = 0;
-    for (int r = 0; r < a.topk_group; ++r) {
-      uint64_t key = (lane < a.n_group && !((kept >> lane) & 1ull))
-                         ? (((uint64_t)f32_order_key(my_gs) << 32) | (uint32_t)(0xffffffffu - (uint32_t)lane))
-                         : 0ull;
-      key = wave_allmax_u64(key);
-      int win = (int)(0xffffffffu - (uint32_t)key);
-      kept |= 1ull << win;
+#undef MERGE2
+    // a group is kept when fewer than topk_group groups beat it (higher score, or the same score
+    // and a lower index): the same set as topk_group rounds of arg-max
+    const uint32_t gkey = f32_order_key(my_gs);
+    int beaten = 0;
+    for (int g = 0; g < a.n_group; ++g) {
+      uint32_t ok = (uint32_t)__builtin_amdgcn_readlane((int)gkey, g);
+      beaten += (ok > gkey || (ok == gkey && g < lane)) ? 1 : 0;
     }
+    const uint64_t kept = __ballot(lane < a.n_group && beaten < a.topk_group);
 #pragma unroll
     for (int j = 0; j < V; ++j) {
       if (in[j] && !((kept >> ge[j]) & 1ull)) c[j] = a.masked_fill_zero ? 0.0f : NEG_INF;
     }
   }
 
-  // ---- K rounds of wave arg-max; ties go to the lower expert id
-  bool taken[V];
+  // ---- K rounds of wave arg-max; ties go to the lower expert id.  A round: each lane's best
+  // remaining key, the wave maximum, then the lowest lane holding it (lanes own ascending ids).
+  uint32_t ck[V];  // order keys of the remaining candidates; 0 once taken (real keys are > 0)
 #pragma unroll
-  for (int j = 0; j < V; ++j) taken[j] = !in[j];
+  for (int j = 0; j < V; ++j) ck[j] = in[j] ? f32_order_key(c[j]) : 0u;
   float my_w = 0.0f;
   int my_id = 0;
   float denom = 0.0f;
   for (int k = 0; k < a.K; ++k) {
-    uint64_t key = 0ull;
+    uint32_t best = ck[0];
+    int bj = 0;
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-      if (!taken[j]) {
-        uint64_t kj = ((uint64_t)f32_order_key(c[j]) << 32) | (uint32_t)(0xffffffffu - (uint32_t)(lane * V + j));
-        key = kj > key ? kj : key;
-      }
+    for (int j = 1; j < V; ++j) {
+      if (ck[j] > best) { best = ck[j]; bj = j; }
     }
-    key = wave_allmax_u64(key);
-    int id = (int)(0xffffffffu - (uint32_t)key);
-    int owner = id / V, sub = id - owner * V;
+    const uint32_t top = wave_allmax_u32(best);
+    const uint64_t holders = __ballot(best == top && best != 0u);
+    const int owner = __ffsll((unsigned long long)holders) - 1;
     float wv = 0.0f;
 #pragma unroll
     for (int j = 0; j < V; ++j) {
-      if (lane == owner && sub == j) {
-        taken[j] = true;
-        wv = a.weight_from_c ? c[j] : s[j];
+      if (bj == j) wv = a.weight_from_c ? c[j] : s[j];
+    }
+    if (lane == owner) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        if (bj == j) ck[j] = 0u;
       }
     }
-    wv = __shfl(wv, owner, WAVE);
+    const int id = owner * V + __builtin_amdgcn_readlane(bj, owner);
+    wv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), owner));
     denom = (k == 0) ? wv : denom + wv;
     if (lane == k) { my_w = wv; my_id = id; }
   }
