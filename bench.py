@@ -31,6 +31,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12       # B/s, MI355X published
 INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/clk x 2.4 GHz = 5.03e15)
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file (scaled by what the same counters read for the 1 GiB copies of --copy-probe); the summaries with
+# the full commands are profiles/decode_gemm1_hbm_traffic.txt and profiles/prefill_gemm1_hbm_traffic.txt.
+MEASURED_TRAFFIC = {"decode": 994_443_000, "prefill": 7_927_757_000}
+
 SHAPES = {
     "decode": dict(T=64, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5, outlier=0.0),
     "prefill": dict(T=8192, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5,
@@ -131,6 +136,8 @@ def main():
     ap.add_argument("--workload", choices=sorted(SHAPES), default="decode")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--weight-sets", type=int, default=2, help="weight copies rotated between steps (cache defeat)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three 1 GiB device copies first (a kernel of known traffic to scale HBM counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's expert share on one GPU; --gpus must be 1 "
@@ -165,6 +172,14 @@ def main():
         return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
                                   (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out)
 
+    if args.copy_probe:
+        src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -178,6 +193,17 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ms = e0.elapsed_time(e1) / args.steps
     ms = max(ms, 0.0)
+
+    # spread of single steps (each bracketed by its own event pair; not part of `value`)
+    nd = min(50, args.steps)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nd)]
+    for i, (a0, a1) in enumerate(evs):
+        a0.record()
+        step(i)
+        a1.record()
+    torch.cuda.synchronize()
+    per = sorted(a0.elapsed_time(a1) * 1e3 for a0, a1 in evs)
+    spread = {"p10": per[int(0.1 * (nd - 1))], "p50": per[(nd - 1) // 2], "p90": per[int(0.9 * (nd - 1))]}
 
     # routing actually produced (rows per local expert) for the byte / op counts
     w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
@@ -215,20 +241,16 @@ def main():
     if args.workload == "decode":
         # weights of every active group + the int8 tokens + the int32 accumulators the kernel writes
         k_alg = active * (H * 2 * I) + T * H + rows_total * 2 * I * 4
-        roof = dict(bound="hbm", kernel="gemm_stream<GEMM1>", achieved=k_alg / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9,
+        roof = dict(bound="hbm", kernel="gemm_stream<1,2,1,4>", achieved=k_alg / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9,
                     unit="GB/s")
     else:
         k_alg = 2 * rows_total * H * 2 * I
-        roof = dict(bound="mfma", kernel="gemm_tile<GEMM1>", achieved=k_alg / (k_ms * 1e-3) / 1e12, peak=INT8_PEAK / 1e12,
+        roof = dict(bound="mfma", kernel="gemm_pipe<1,4>", achieved=k_alg / (k_ms * 1e-3) / 1e12, peak=INT8_PEAK / 1e12,
                     unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["kernel_us"] = k_ms * 1e3
     roof["algorithmic_per_launch"] = k_alg
-    roof["traffic"] = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            roof["traffic"] = json.load(f).get(args.workload)
+    roof["traffic"] = MEASURED_TRAFFIC.get(args.workload)
 
     result = {
         "metric": "moe_layer_latency", "value": ms * 1e3, "unit": "us", "n_gpus": 1, "steps": args.steps,
@@ -239,7 +261,7 @@ def main():
                    "tokens": T, "rows_routed": rows_routed, "active_groups": active, "weight_sets": len(sets)},
         "layer": {"algorithmic_bytes": layer_bytes, "algorithmic_ops": layer_ops,
                   "hbm_frac": layer_bytes / (ms * 1e-3) / HBM_PEAK, "int8_frac": layer_ops / (ms * 1e-3) / INT8_PEAK,
-                  "host_wall_ms_per_step": wall_ms},
+                  "host_wall_ms_per_step": wall_ms, "single_step_us": spread},
         "roofline": roof,
     }
     if not args.no_cpu:
