@@ -253,26 +253,48 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
 template <int PMAX>
 __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __restrict__ hq, float* __restrict__ hs) {
   __shared__ float red[4];
-  __shared__ int s_group;
-  const int64_t m = blockIdx.x;
-  // group g with offsets[g] <= m < offsets[g+1] (rows from offsets[G] on: the extra group); one
-  // thread per group looks, so the lookup costs one round trip to memory
+  __shared__ int s_group, s_first;
+  const int64_t m = blockIdx.x;  // < M_cap: the row's partial sums exist (unused rows hold anything)
+  const int I = a.N / 2;
+  // everything that does not depend on the row's group is requested first: the partial sums and
+  // the row's source assignment; the group lookup (one thread per group) overlaps with them
+  const size_t plane = (size_t)a.M_cap * a.N;
+  const int32_t* prow = a.part + (size_t)m * a.N;
+  int ag[PMAX], au[PMAX];
+#pragma unroll
+  for (int i = 0; i < PMAX; ++i) {
+    const int n = threadIdx.x + i * 256;
+    ag[i] = 0;
+    au[i] = 0;
+    if (n < I) {
+      for (int sp = 0; sp < a.S; ++sp) {
+        ag[i] += prow[sp * plane + n];
+        au[i] += prow[sp * plane + I + n];
+      }
+    }
+  }
+  int src = 0;
+  if (a.sorted_src != nullptr && m < (int64_t)a.T * a.K) src = a.sorted_src[m];
   if (threadIdx.x == 0) s_group = -1;
   __syncthreads();
   for (int g = threadIdx.x; g <= a.G; g += 256) {
     const int64_t lo = a.offsets[g];
     const int64_t hi = (g < a.G) ? (int64_t)a.offsets[g + 1] : lo + a.extra_rows;
-    if (m >= lo && m < hi) s_group = g;
+    if (m >= lo && m < hi) {
+      s_group = g;
+      s_first = (int)lo;
+    }
   }
   __syncthreads();
   if (s_group < 0) return;  // past the last row
   const int g = s_group;
-  const int I = a.N / 2;
   const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
-  const float ts = a.a_scale[source_row<1>(a, g, (int)m)];
+  int token;  // row of the activation matrix this row came from (what source_row<1> computes)
+  if (g >= a.G) token = (int)m - s_first;
+  else if (a.sorted_src == nullptr) token = (int)m;
+  else token = (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? src / a.K : src % a.T;
+  const float ts = a.a_scale[token];
   const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
-  const size_t plane = (size_t)a.M_cap * a.N;
-  const int32_t* prow = a.part + (size_t)m * a.N;
   float y[PMAX];
   float amax = 0.0f;
 #pragma unroll
@@ -280,17 +302,12 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
     const int n = threadIdx.x + i * 256;
     y[i] = 0.0f;
     if (n < I) {
-      int ag = 0, au = 0;
-      for (int sp = 0; sp < a.S; ++sp) {
-        ag += prow[sp * plane + n];
-        au += prow[sp * plane + I + n];
-      }
       if (a.acc_dbg) {
-        a.acc_dbg[(size_t)m * a.N + n] = ag;
-        a.acc_dbg[(size_t)m * a.N + I + n] = au;
+        a.acc_dbg[(size_t)m * a.N + n] = ag[i];
+        a.acc_dbg[(size_t)m * a.N + I + n] = au[i];
       }
-      float dg = ((float)ag * wsc[n]) * ts;
-      float du = ((float)au * wsc[I + n]) * ts;
+      float dg = ((float)ag[i] * wsc[n]) * ts;
+      float du = ((float)au[i] * wsc[I + n]) * ts;
       if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
       float yv = silu_spec(dg) * du;
       if (bf) yv = round_bf16(yv);

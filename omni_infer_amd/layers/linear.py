@@ -33,6 +33,12 @@ class ReplicatedLinear(nn.Module):
             return torch.nn.functional.linear(x, self.weight), None
         return self.quant_method.apply_weights(self, x, None), None
 
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor) -> None:
+        """vLLM's ``ReplicatedLinear.weight_loader``: a whole-parameter copy; shapes must agree."""
+        if param.data.shape != loaded_weight.shape:
+            raise RuntimeError("param_data.shape != loaded_weight.shape")
+        param.data.copy_(loaded_weight)
+
 
 class MergedReplicatedLinear(ReplicatedLinear):
     """gate_proj and up_proj stacked along the output dim (linear.py:620-762)."""
@@ -41,3 +47,26 @@ class MergedReplicatedLinear(ReplicatedLinear):
                  params_dtype: Optional[torch.dtype] = None, prefix: str = "", device=None):
         self.output_sizes = output_sizes
         super().__init__(input_size, sum(output_sizes), bias, quant_config, params_dtype, prefix, device)
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor,
+                      loaded_shard_id: Optional[int] = None) -> None:
+        """linear.py:639-762 for parameters stacked along dim 0 (weights [out, in], per-channel
+        scales and offsets [out, 1]): shard ``i`` fills rows ``sum(output_sizes[:i])`` onwards;
+        without a shard id a fused checkpoint tensor is split over the shards."""
+        if loaded_shard_id is None:
+            if param.data.shape[0] != loaded_weight.shape[0]:
+                raise RuntimeError("param_data.shape != loaded_weight.shape")
+            offset = 0
+            for i, size in enumerate(self.output_sizes):
+                self.weight_loader(param, loaded_weight.narrow(0, offset, size), i)
+                offset += size
+            return
+        if loaded_shard_id >= len(self.output_sizes):
+            raise RuntimeError("loaded_shard_id >= len(self.output_sizes)")
+        offset = sum(self.output_sizes[:loaded_shard_id])
+        size = self.output_sizes[loaded_shard_id]
+        dst = param.data.narrow(0, offset, size)
+        src = loaded_weight.narrow(0, 0, size)
+        if dst.shape != src.shape:
+            raise RuntimeError("param_data.shape != loaded_weight.shape")
+        dst.copy_(src)
