@@ -104,6 +104,21 @@ int omni_dynamic_quant(const void* x, int in_dtype, int64_t rows, int cols, int6
                        void* stream);
 
 /*
+ * Residual add + RMSNorm (+ per-token dynamic quantisation of the result) in one pass: the producer
+ * in front of the MoE block.  Replaces RMSNorm.forward (omni/models/common/layers/layernorm.py:13-32):
+ * npu_add_rms_norm(x, residual, weight, eps) followed, under quant_symbol, by npu_dynamic_quant
+ * (:21-25; call sites deepseek_v3.py:219-220,233-235); residual == NULL gives npu_rms_norm (:28-32).
+ * x, residual, weight, residual_out, y: bf16; rows x H row-major, H % 8 == 0, H <= 8192.
+ *   s = float(x) + float(residual); residual_out = bf16(s);
+ *   y = bf16((s / sqrt(mean(s*s) + eps)) * weight)     (fixed summation order, see csrc/norm.hip)
+ *   scale = max|y| / 127, q = rint(y / scale)           (q/scale optional, together)
+ * Any of residual_out, y, q may be NULL (at least one output).  residual_out may be residual itself.
+ */
+int omni_add_rms_norm_quant(const void* x_bf16, const void* residual_bf16, const void* weight_bf16, int64_t rows,
+                            int H, float eps, void* residual_out_bf16, void* y_bf16, int8_t* q, float* scale,
+                            void* stream);
+
+/*
  * Sort (token, k) assignments by expert.  Replaces torch_npu.npu_moe_init_routing +
  * npu_moe_compute_expert_tokens (compressed_tensors_moe.py:235-237) and
  * npu_moe_init_routing_v2 with active_expert_range (fused_moe.py:514-515, :607-618).

@@ -101,6 +101,32 @@ def npu_dynamic_quant(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q.view(shape), s.view(shape[:-1])
 
 
+def add_rms_norm_quant(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                       want_y: bool = True, want_quant: bool = False, inplace_residual: bool = False):
+    """Stands in for ``npu_add_rms_norm`` / ``npu_rms_norm`` and, with ``want_quant``, the
+    ``npu_dynamic_quant`` that follows it (omni/models/common/layers/layernorm.py:13-32).
+    Returns (y or None, residual_out or None, x_int8 or None, pertoken_scale or None)."""
+    _need_gpu(x, weight)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or (residual is not None and residual.dtype != torch.bfloat16):
+        raise ValueError("add_rms_norm_quant: bf16 tensors only")
+    shape = x.shape
+    H = shape[-1]
+    x2 = x.reshape(-1, H).contiguous()
+    rows = x2.shape[0]
+    r2 = residual.reshape(-1, H).contiguous() if residual is not None else None
+    res_out = None
+    if r2 is not None:
+        res_out = r2 if inplace_residual else torch.empty_like(r2)
+    y = torch.empty_like(x2) if want_y else None
+    q = torch.empty(rows, H, dtype=torch.int8, device=x.device) if want_quant else None
+    sc = torch.empty(rows, dtype=torch.float32, device=x.device) if want_quant else None
+    rc = L.lib().omni_add_rms_norm_quant(_ptr(x2), _ptr(r2), _ptr(weight.contiguous()), rows, H, float(eps),
+                                         _ptr(res_out), _ptr(y), _ptr(q), _ptr(sc), _stream())
+    L.check(rc, "omni_add_rms_norm_quant")
+    return (y.view(shape) if y is not None else None, res_out.view(shape) if res_out is not None else None,
+            q.view(shape) if q is not None else None, sc.view(shape[:-1]) if sc is not None else None)
+
+
 # ----------------------------------------------------------------------------- permutation
 class Permutation:
     """Result of sorting the (token, k) assignments by local expert."""

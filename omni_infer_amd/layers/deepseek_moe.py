@@ -137,6 +137,8 @@ class DeepseekMoE(nn.Module):
                       self.shared_experts.down_proj.input_size == self.experts.intermediate_size_per_partition)
         if self.fused and allgather_ep and same_width and self.quant_symbol:
             return self._forward_fused(hidden_states), residual
+        if isinstance(hidden_states, dict):
+            hidden_states = hidden_states["x"]
         return self._forward_norm_ops(hidden_states, attn_metadata), residual
 
     def _forward_norm_ops(self, hidden_states, attn_metadata):
@@ -157,6 +159,11 @@ class DeepseekMoE(nn.Module):
         return final
 
     def _forward_fused(self, hidden_states):
+        # a dict from RMSNorm.forward_moe_input carries the tokens already quantised
+        x_int8 = pertoken_scale = None
+        if isinstance(hidden_states, dict):
+            x_int8, pertoken_scale = hidden_states["x_int8"], hidden_states["pertoken_scale"]
+            hidden_states = hidden_states["x"]
         topk_weights, topk_ids = self._route(hidden_states)
         e = self.experts
         lo = self.global_rank * self.local_expert_num
@@ -169,6 +176,7 @@ class DeepseekMoE(nn.Module):
                                                                e.intermediate_size_per_partition, int(shared is not None))
         if self._workspace is None or self._workspace.numel() < need:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=hidden_states.device)
-        return ops.moe_w8a8_layer(hidden_states, None, topk_weights, topk_ids, lo, lo + self.local_expert_num,
+        x_in = hidden_states if x_int8 is None else x_int8
+        return ops.moe_w8a8_layer(x_in, pertoken_scale, topk_weights, topk_ids, lo, lo + self.local_expert_num,
                                   e.w13_weight, e.w13_weight_scale, e.w2_weight, e.w2_weight_scale.float(), shared,
                                   H=e.hidden_size, I=e.intermediate_size_per_partition, workspace=self._workspace)

@@ -45,6 +45,11 @@ tests/test_oracle_pins.py):
 * dequant_swiglu_quant, grouped_matmul_dequant, finalize ... closed forms in
   float64, and the end-to-end dense brute force (every token through every
   selected expert without any permutation).
+* add_rms_norm / add_rms_norm_dynamic_quant (the producer in front of the
+  block) ... torch.nn.functional.rms_norm in float64 (library routine) within
+  one bf16 step, closed forms on constant and zero rows, power-of-two scale
+  invariance, unit RMS, the quantisation invariants; its square root against
+  numpy's (tests/test_norm.py).
 
 Parity unpinned by the reference itself: the reference holds no test, golden
 vector or fixture for this path, and the rounding mode, zero-row behaviour,
@@ -265,6 +270,63 @@ def dynamic_quant(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     q = torch.where((s > 0).unsqueeze(-1), q, torch.zeros_like(q))
     q = torch.clamp(q, -128, 127).to(torch.int8)
     return q, s
+
+
+# --------------------------------------------------------------------------
+# Residual add + RMSNorm (+ dynamic quant): the producer in front of the block
+# --------------------------------------------------------------------------
+def _sqrt_rn(v: torch.Tensor) -> torch.Tensor:
+    """Correctly rounded fp32 square root.  torch's vectorised fp32 sqrt on x86 is off by one unit in
+    the last place for about 0.7 % of inputs (checked against numpy and against the rounded fp64 root);
+    the fp64 root rounded to fp32 is the correctly rounded result (53 >= 2*24 + 2 bits)."""
+    return torch.sqrt(v.to(torch.float64)).to(F32)
+
+
+def add_rms_norm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float
+                 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """``RMSNorm.forward`` (omni/models/common/layers/layernorm.py:13-32):
+    ``npu_add_rms_norm(x, residual, weight, eps)`` -> (y, residual_out), or
+    ``npu_rms_norm(x, weight, eps)`` when there is no residual.
+
+    s = float(x) + float(residual); residual_out = s rounded to the input dtype;
+    y = ((s * r) * float(weight)) rounded to the input dtype, r = 1 / sqrt(mean(s*s) + eps) with a
+    correctly rounded root and a true division.
+    The mean's sum has a fixed order: the row is cut into vectors of 8 elements; slot t of 256
+    owns vectors t, t+256, ... and adds their squares in index order; the 64 slots of each of the
+    four groups are combined by the xor butterfly (1..32) and the groups as ((g0+g1)+g2)+g3.
+    """
+    dt = x.dtype
+    T, H = x.shape
+    assert H % 8 == 0
+    s = x.to(F32)
+    res_out = None
+    if residual is not None:
+        s = s + residual.to(F32)
+        res_out = s.to(dt)
+    nvec = H // 8
+    rounds = (nvec + 255) // 256
+    sq = torch.zeros(T, rounds * 256 * 8, dtype=F32)
+    sq[:, :H] = s * s
+    sq = sq.view(T, rounds, 256, 8)
+    acc = torch.zeros(T, 256, dtype=F32)
+    for i in range(rounds):
+        for j in range(8):
+            acc = acc + sq[:, i, :, j]      # absent vectors add exact zeros
+    groups = [_butterfly_sum64(acc[:, 64 * g:64 * g + 64].contiguous()) for g in range(4)]
+    total = ((groups[0] + groups[1]) + groups[2]) + groups[3]
+    mean = total / _c(float(H))
+    r = _c(1.0) / _sqrt_rn(mean + _c(eps))
+    y = ((s * r.unsqueeze(-1)) * weight.to(F32)).to(dt)
+    return y, res_out
+
+
+def add_rms_norm_dynamic_quant(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float):
+    """``RMSNorm.forward(..., quant_symbol=True)`` (layernorm.py:21-25): the normalised
+    tensor, in the model dtype, goes through ``npu_dynamic_quant``.
+    Returns (x_int8, pertoken_scale, residual_out)."""
+    y, res_out = add_rms_norm(x, residual, weight, eps)
+    q, sc = dynamic_quant(y)
+    return q, sc, res_out
 
 
 # --------------------------------------------------------------------------
