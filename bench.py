@@ -128,12 +128,75 @@ def cpu_baseline(cfg, ws, x, logits, bias, sample_tokens):
     return dt, out
 
 
+def bench_norm(args):
+    """Secondary workload: the producer in front of the block (residual add + RMSNorm + dynamic quant,
+    all three outputs) on 8192 x 7168 bf16 rows.  One step = one launch; input sets are rotated so that
+    the rows come from HBM."""
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+    T, H, eps = 8192, 7168, 1e-6
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    nsets = 4
+    xs = [torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16) for _ in range(nsets)]
+    rs = [torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16) for _ in range(nsets)]
+    w = (1.0 + 0.1 * torch.randn(H, generator=g, device=dev)).to(torch.bfloat16)
+    y = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    ro = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    q = torch.empty(T, H, dtype=torch.int8, device=dev)
+    sc = torch.empty(T, dtype=torch.float32, device=dev)
+    lib, st = L.lib(), torch.cuda.current_stream().cuda_stream
+
+    def step(i):
+        rc = lib.omni_add_rms_norm_quant(xs[i % nsets].data_ptr(), rs[i % nsets].data_ptr(), w.data_ptr(), T, H, eps,
+                                         ro.data_ptr(), y.data_ptr(), q.data_ptr(), sc.data_ptr(), st)
+        L.check(rc, "omni_add_rms_norm_quant")
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    alg = T * H * (2 + 2 + 2 + 2 + 1) + T * 4 + H * 2     # x, residual in; residual, y, int8 out; scales; weight
+    result = {"metric": "add_rms_norm_quant_latency", "value": ms * 1e3, "unit": "us", "n_gpus": 1, "steps": args.steps,
+              "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak",
+              "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+              "config": {"workload": f"residual add + RMSNorm + per-token int8 quantisation, {T} x {H} bf16 rows, "
+                                     "outputs: residual, normalised rows, int8 rows + scales", "rows": T, "H": H},
+              "roofline": {"bound": "hbm", "kernel": "add_rms_norm_quant_kernel", "achieved": alg / (ms * 1e-3) / 1e9,
+                           "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": alg / (ms * 1e-3) / HBM_PEAK,
+                           "kernel_us": ms * 1e3, "algorithmic_per_launch": alg, "traffic": None}}
+    if not args.no_cpu:
+        from oracle import moe_oracle as O
+        torch.set_num_threads(os.cpu_count() or 1)
+        n = 1024
+        xc, rc_, wc = xs[0][:n].cpu(), rs[0][:n].cpu(), w.cpu()
+        O.add_rms_norm_dynamic_quant(xc, rc_, wc, eps)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            qr, sr, rr = O.add_rms_norm_dynamic_quant(xc, rc_, wc, eps)
+        dt = (time.perf_counter() - t0) / 3
+        step(0)
+        torch.cuda.synchronize()
+        result["cpu_baseline"] = {"value": dt * 1e6 * (T / n), "unit": "us", "cores": torch.get_num_threads(),
+                                  "kind": "port", "sample": f"oracle on the first {n} of {T} rows, scaled by rows",
+                                  "gpu_vs_oracle_bit_exact": bool(torch.equal(q[:n].cpu(), qr) and
+                                                                  torch.equal(sc[:n].cpu(), sr) and
+                                                                  torch.equal(ro[:n].cpu(), rr))}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=sorted(SHAPES), default="decode")
+    ap.add_argument("--workload", choices=sorted(SHAPES) + ["norm"], default="decode",
+                    help="decode (default, the headline metric) / prefill: the MoE layer; norm: the RMSNorm+quant producer")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--weight-sets", type=int, default=2, help="weight copies rotated between steps (cache defeat)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -146,6 +209,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "norm":
+        return bench_norm(args)
 
     from omni_infer_amd import _lib as L
     from omni_infer_amd import hip_ops as ops

@@ -34,12 +34,13 @@ struct CombineArgs {
   uint16_t* out;
 };
 
-template <int DT>
+// STREAM: the row is read once and not again (expert rows), so it need not stay in the caches
+template <int DT, bool STREAM = false>
 __device__ __forceinline__ void load4(const void* base, size_t row, int H, int c, int ncol, float* v) {
   if constexpr (DT == OMNI_DT_F32) {
     const float* p = (const float*)base + row * H + c;
     if (ncol == 4) {
-      v4f t = *(const v4f*)p;
+      v4f t = STREAM ? __builtin_nontemporal_load((const v4f*)p) : *(const v4f*)p;
       v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
     } else {
       for (int j = 0; j < 4; ++j) v[j] = j < ncol ? p[j] : 0.0f;
@@ -47,7 +48,7 @@ __device__ __forceinline__ void load4(const void* base, size_t row, int H, int c
   } else {
     const uint16_t* p = (const uint16_t*)base + row * H + c;
     if (ncol == 4) {
-      v2i t = *(const v2i*)p;
+      v2i t = STREAM ? __builtin_nontemporal_load((const v2i*)p) : *(const v2i*)p;
       v[0] = bf16_to_f32((uint16_t)((uint32_t)t[0] & 0xffffu));
       v[1] = bf16_to_f32((uint16_t)((uint32_t)t[0] >> 16));
       v[2] = bf16_to_f32((uint16_t)((uint32_t)t[1] & 0xffffu));
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
   if (a.init) load4<OMNI_DT_BF16>(a.init, (size_t)n, a.H, c, ncol, acc);
   for (int j = 0; j < cnt; ++j) {
     float v[4];
-    load4<DT>(a.rows, (size_t)s_slot[j], a.H, c, ncol, v);
+    load4<DT, true>(a.rows, (size_t)s_slot[j], a.H, c, ncol, v);
     const float wv = s_w[j];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -58,13 +58,14 @@ __global__ __launch_bounds__(256) void add_rms_norm_quant_kernel(NormArgs a) {
   for (int i = 0; i < NORM_MAXV; ++i) {
     const int vi = threadIdx.x + i * 256;
     if (vi < nvec) {
-      unpack8(*(const v4i*)(xr + (size_t)vi * 8), s[i]);
+      unpack8(__builtin_nontemporal_load((const v4i*)(xr + (size_t)vi * 8)), s[i]);  // read once
       if (rr) {
         float t[8];
-        unpack8(*(const v4i*)(rr + (size_t)vi * 8), t);
+        unpack8(__builtin_nontemporal_load((const v4i*)(rr + (size_t)vi * 8)), t);
 #pragma unroll
         for (int j = 0; j < 8; ++j) s[i][j] = s[i][j] + t[j];
-        if (a.residual_out) *(v4i*)(a.residual_out + r * a.H + (size_t)vi * 8) = pack8(s[i]);
+        if (a.residual_out)  // next read: the following layer's norm, long after it left the caches
+          __builtin_nontemporal_store(pack8(s[i]), (v4i*)(a.residual_out + r * a.H + (size_t)vi * 8));
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
