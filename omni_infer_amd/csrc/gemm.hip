@@ -416,7 +416,9 @@ __device__ __forceinline__ int tile32_row(int lane, int i) { return 8 * (i >> 2)
 
 // WN = 2: 256 threads, tile 256 x 128, two blocks per CU.  WN = 4: 512 threads, tile 256 x 256, one block
 // per CU (a third fewer operand bytes through the vector memory path per MFMA).
-template <int KIND, int WN>
+// BF (GEMM1 only): round gate, up and their product to bf16 (the numerics of the reference's
+// unfused bf16 path); a template parameter so that the fp32 path carries none of that arithmetic.
+template <int KIND, int WN, bool BF>
 __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int BM = 256;
@@ -510,7 +512,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
   uint16_t* stage16 = (uint16_t*)(w < 3 ? sa0 : (w < 6 ? sa1 : sa2)) + (w % 3) * (32 * OUT_PITCH);
   if (bf16_out) __syncthreads();  // every wavefront is done reading the last stage
-  const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+  constexpr bool bf = BF;
   float wsc_g[2];
   int ncol[2];
   if constexpr (KIND == 1) {
@@ -761,10 +763,12 @@ void launch_tile(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
   int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
   if (tile_wn(KIND, units) == 4) {
     dim3 grid((unsigned)(units / ((KIND == 1) ? 8 : 16)), (unsigned)mblocks), block(512);
-    hipLaunchKernelGGL((gemm_pipe<KIND, 4>), grid, block, 0, st, a);
+    if (KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE)) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_pipe<KIND, 4, false>), grid, block, 0, st, a);
   } else {
     dim3 grid((unsigned)(units / ((KIND == 1) ? 4 : 8)), (unsigned)mblocks), block(256);
-    hipLaunchKernelGGL((gemm_pipe<KIND, 2>), grid, block, 0, st, a);
+    if (KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE)) hipLaunchKernelGGL((gemm_pipe<KIND, 2, KIND == 1>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_pipe<KIND, 2, false>), grid, block, 0, st, a);
   }
 }
 
