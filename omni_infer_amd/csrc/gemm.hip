@@ -507,10 +507,11 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // ---- epilogue, one 32-row tile at a time
   const int c32 = lane & 31;
   // bf16 rows of GEMM2 are transposed through LDS (the stage buffers are free now): a private
-  // 32 x 64 piece per wavefront, rows padded to 144 bytes; three wavefronts share a stage buffer
-  constexpr int OUT_PITCH = 72;  // uint16 elements
+  // 32 x 64 piece per wavefront, rows padded to 192 bytes (48 dwords: the two rows a half-wavefront
+  // writes at once then fall into disjoint banks); two wavefronts share a stage buffer
+  constexpr int OUT_PITCH_DW = 48;
   const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
-  uint16_t* stage16 = (uint16_t*)(w < 3 ? sa0 : (w < 6 ? sa1 : sa2)) + (w % 3) * (32 * OUT_PITCH);
+  uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * (32 * OUT_PITCH_DW);
   if (bf16_out) __syncthreads();  // every wavefront is done reading the last stage
   constexpr bool bf = BF;
   float wsc_g[2];
@@ -524,40 +525,73 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   }
   wsc_g[0] = wsc[ncol[0]];
   wsc_g[1] = wsc[ncol[1]];
+  if (bf16_out) {
+    if constexpr (KIND == 2) {
+      const int odd = c32 & 1;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int tile_r0 = wm * 128 + mt * 32;
-    if (tile_r0 < nrows) {
+      for (int mt = 0; mt < 4; ++mt) {
+        const int tile_r0 = wm * 128 + mt * 32;
+        if (tile_r0 < nrows) {
+          // accumulator entries i, i+1 (i even) are rows r, r+1 of the same channel; neighbouring
+          // lanes hold neighbouring channels.  One pack + one lane exchange gives every lane a
+          // dword of two neighbouring channels: even lanes for row r, odd lanes for row r+1.
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int rr = tile_r0 + tile32_row(lane, i);
-        const bool ok = rr < nrows;
-        const size_t m = (size_t)(row0 + rr);
-        const float ts = row_scale[rr];
-        if constexpr (KIND == 1) {
-          if (ok) {
-            float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
-            float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
-            if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
-            float yv = silu_spec(dg) * du;
-            if (bf) yv = round_bf16(yv);
-            __builtin_nontemporal_store(yv, &a.y[m * I + ncol[0]]);  // read once, by the row quantiser
-            if (a.acc_dbg) {
-              a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
-              a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
+          for (int i = 0; i < 16; i += 2) {
+            const int r = tile32_row(lane, i);
+            const float ts0 = row_scale[tile_r0 + r], ts1 = row_scale[tile_r0 + r + 1];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              const float o0 = ((float)acc[mt][t][i] * wsc_g[t]) * ts0;
+              const float o1 = ((float)acc[mt][t][i + 1] * wsc_g[t]) * ts1;
+              const uint32_t mine = f32x2_to_bf16x2(o0, o1);
+              const uint32_t theirs = (uint32_t)xchg_i<1>((int)mine);
+              const uint32_t out = odd ? ((theirs >> 16) | (mine & 0xffff0000u)) : ((mine & 0xffffu) | (theirs << 16));
+              stage32[(r + odd) * OUT_PITCH_DW + t * 16 + (c32 >> 1)] = out;
+              if (a.acc_dbg) {
+#pragma unroll
+                for (int d = 0; d < 2; ++d)
+                  if (tile_r0 + r + d < nrows)
+                    a.acc_dbg[(size_t)(row0 + tile_r0 + r + d) * (size_t)a.N + ncol[t]] = acc[mt][t][i + d];
+              }
             }
           }
-        } else {
-          if (bf16_out) {
-            // through LDS: the tile's 64 channels of a row become one 128-byte line
-            const float o0 = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
-            const float o1 = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
-            const uint32_t pk = f32x2_to_bf16x2(o0, o1);
-            stage16[tile32_row(lane, i) * OUT_PITCH + c32] = (uint16_t)(pk & 0xffffu);
-            stage16[tile32_row(lane, i) * OUT_PITCH + 32 + c32] = (uint16_t)(pk >> 16);
-            if (ok && a.acc_dbg) {
-              a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
-              a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
+          // the wavefront wrote its 32 x 64 piece; now 8 lanes per row store 16 bytes each
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = j * 8 + (lane >> 3);
+            const int rr = tile_r0 + r;
+            v4i v = *(const v4i*)(stage32 + r * OUT_PITCH_DW + (lane & 7) * 4);
+            if (rr < nrows)  // read once, by the combine
+              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int tile_r0 = wm * 128 + mt * 32;
+      if (tile_r0 < nrows) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int rr = tile_r0 + tile32_row(lane, i);
+          const bool ok = rr < nrows;
+          const size_t m = (size_t)(row0 + rr);
+          const float ts = row_scale[rr];
+          if constexpr (KIND == 1) {
+            if (ok) {
+              float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
+              float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
+              if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+              float yv = silu_spec(dg) * du;
+              if (bf) yv = round_bf16(yv);
+              __builtin_nontemporal_store(yv, &a.y[m * I + ncol[0]]);  // read once, by the row quantiser
+              if (a.acc_dbg) {
+                a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
+                a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
+              }
             }
           } else if (ok) {
 #pragma unroll
@@ -567,21 +601,6 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
               if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + ncol[t]] = acc[mt][t][i];
             }
           }
-        }
-      }
-      if constexpr (KIND == 2) {
-        if (bf16_out) {
-          // the wavefront wrote its 32 x 64 piece; now 8 lanes per row store 16 bytes each
-          __builtin_amdgcn_wave_barrier();
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int r = j * 8 + (lane >> 3);
-            const int rr = tile_r0 + r;
-            v4i v = *(const v4i*)(stage16 + r * OUT_PITCH + (lane & 7) * 8);
-            if (rr < nrows)  // read once, by the combine
-              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
-          }
-          __builtin_amdgcn_wave_barrier();
         }
       }
     }
