@@ -212,18 +212,31 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
   const int8_t* xq = (const int8_t*)x;
   const float* xs = x_scale_in;
   int rc;
-  if (x_dtype != -1) {
-    rc = omni_dynamic_quant(x, x_dtype, T, H, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), stream);
-    if (rc) return rc;
-    xq = (const int8_t*)(ws + L.x_q);
-    xs = (const float*)(ws + L.x_s);
-  }
   int32_t* sorted_src = (int32_t*)(ws + L.sorted_src);
   int32_t* src_to_dst = (int32_t*)(ws + L.src_to_dst);
   int32_t* offsets = (int32_t*)(ws + L.offsets);
-  rc = omni_moe_permute(topk_ids, T, K, lo, hi, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts),
-                        offsets, ws + L.perm_ws, L.perm_bytes, stream);
-  if (rc) return rc;
+  bool sorted = false;
+  if (x_dtype != -1) {
+    // the quantisation and the sort do not depend on each other: one launch when both are small
+    rc = 1;
+    if (x_dtype == OMNI_DT_BF16)
+      rc = omni_quant_permute_fused(x, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), topk_ids, K, lo, hi,
+                                    OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts), offsets,
+                                    stream);
+    if (rc < 0) return rc;
+    sorted = rc == 0;
+    if (!sorted) {
+      rc = omni_dynamic_quant(x, x_dtype, T, H, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), stream);
+      if (rc) return rc;
+    }
+    xq = (const int8_t*)(ws + L.x_q);
+    xs = (const float*)(ws + L.x_s);
+  }
+  if (!sorted) {
+    rc = omni_moe_permute(topk_ids, T, K, lo, hi, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts),
+                          offsets, ws + L.perm_ws, L.perm_bytes, stream);
+    if (rc) return rc;
+  }
   const int extra = with_shared ? T : 0;
   rc = omni_moe_gemm1_swiglu_quant(xq, xs, sorted_src, OMNI_IDX_TOKEN_MAJOR, T, K, w13_packed, w13_scale, sh13_packed,
                                    sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),

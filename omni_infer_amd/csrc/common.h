@@ -29,6 +29,11 @@ void omni_set_error(const char* fmt, ...);
     if (e__ != hipSuccess) OMNI_FAIL(OMNI_E_LAUNCH, "%s: %s", what, hipGetErrorString(e__)); \
   } while (0)
 
+// library-internal: bf16 row quantisation and assignment sort in one launch (permute.hip); 1 = not applicable
+int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float* scale, const int32_t* topk_ids, int K,
+                             int lo, int hi, int idx_mode, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
+                             int32_t* offsets, void* stream);
+
 // ---------------------------------------------------------------- specified transcendental
 // exp with a fixed operation sequence: clamp to [-87, 87], Cody-Waite reduction by ln2 split in
 // two constants, the Cephes expf polynomial by Horner, scaling by 2^n through the exponent field.

@@ -9,6 +9,7 @@
 // Small inputs (<= 4096 assignments) are sorted by one block in one launch; larger ones take a
 // count launch, a one-block scan launch and a scatter launch.
 #include "common.h"
+#include "quant_rows.h"
 
 namespace {
 
@@ -110,7 +111,7 @@ __device__ __forceinline__ void wave0_excl_scan(const int* tot, int* off, int nb
   }
 }
 
-__global__ __launch_bounds__(256) void permute_single(PermArgs a) {
+__device__ __forceinline__ void permute_single_body(const PermArgs& a) {
   __shared__ int whist[4][NB];
   __shared__ int lrank[CH_SINGLE];
   __shared__ int tot[NB];
@@ -128,6 +129,19 @@ __global__ __launch_bounds__(256) void permute_single(PermArgs a) {
   }
   if (threadIdx.x == 0) a.offsets[a.G] = off[a.G];
   scatter_chunk(a, 0, a.n, passes, whist, lrank, off);
+}
+
+__global__ __launch_bounds__(256) void permute_single(PermArgs a) { permute_single_body(a); }
+
+// One launch for the two independent first steps of a small layer call: blocks [0, rows) quantise
+// one bf16 token row each, the last block sorts the assignments.
+template <int MAXV>
+__global__ __launch_bounds__(256) void quant_permute_small(const void* __restrict__ x, int64_t rows, int cols,
+                                                           int8_t* __restrict__ q, float* __restrict__ scale,
+                                                           PermArgs a) {
+  __shared__ float red[4];
+  if ((int64_t)blockIdx.x < rows) quant_row_vec_body<OMNI_DT_BF16, MAXV>(x, (int64_t)blockIdx.x, cols, cols, q, scale, red);
+  else permute_single_body(a);
 }
 
 __global__ __launch_bounds__(256) void permute_count(PermArgs a) {
@@ -241,6 +255,25 @@ extern "C" int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, i
   hipLaunchKernelGGL(permute_scan, dim3(1), dim3(256), 0, st, a);
   hipLaunchKernelGGL(permute_scatter, dim3(a.nblk), dim3(256), 0, st, a);
   OMNI_CHECK_LAUNCH("permute");
+  return OMNI_OK;
+}
+
+// Internal to the library (the whole-layer entry uses it): quantise bf16 rows and sort the
+// assignments in one launch.  Returns 1 without launching when the shapes do not fit that kernel.
+int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float* scale, const int32_t* topk_ids, int K,
+                             int lo, int hi, int idx_mode, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
+                             int32_t* offsets, void* stream) {
+  const int G = hi - lo;
+  const int64_t n = (int64_t)T * K;
+  if (T <= 0 || n > CH_SINGLE || G > GMAX || H % 8 != 0 || H > 8 * 256 * 4) return 1;
+  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((size_t)H * 2) % 16 != 0) return 1;
+  PermArgs a{topk_ids, (int)n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, nullptr, 0};
+  dim3 grid((unsigned)T + 1), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (H <= 8 * 256 * 1) hipLaunchKernelGGL(quant_permute_small<1>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
+  else if (H <= 8 * 256 * 2) hipLaunchKernelGGL(quant_permute_small<2>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
+  else hipLaunchKernelGGL(quant_permute_small<4>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
+  OMNI_CHECK_LAUNCH("quant_permute");
   return OMNI_OK;
 }
 
