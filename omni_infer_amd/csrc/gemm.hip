@@ -250,9 +250,10 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
 // quantises.  Each thread keeps its y values in registers between the two passes (PMAX pairs,
 // I <= 256*PMAX); nothing but the int8 row and its scale is written.
 // =====================================================================================
-template <int PMAX>
-__global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __restrict__ hq, float* __restrict__ hs) {
-  __shared__ float red[4];
+// NTH threads per row (a multiple of 64, at most 1024); a thread owns PMAX channel pairs
+template <int PMAX, int NTH>
+__global__ __launch_bounds__(NTH) void swiglu_quant_rows(GemmArgs a, int8_t* __restrict__ hq, float* __restrict__ hs) {
+  __shared__ float red[NTH / WAVE];
   __shared__ int s_group, s_first;
   const int64_t m = blockIdx.x;  // < M_cap: the row's partial sums exist (unused rows hold anything)
   const int I = a.N / 2;
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
   int ag[PMAX], au[PMAX];
 #pragma unroll
   for (int i = 0; i < PMAX; ++i) {
-    const int n = threadIdx.x + i * 256;
+    const int n = threadIdx.x + i * NTH;
     ag[i] = 0;
     au[i] = 0;
     if (n < I) {
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
   if (a.sorted_src != nullptr && m < (int64_t)a.T * a.K) src = a.sorted_src[m];
   if (threadIdx.x == 0) s_group = -1;
   __syncthreads();
-  for (int g = threadIdx.x; g <= a.G; g += 256) {
+  for (int g = threadIdx.x; g <= a.G; g += NTH) {
     const int64_t lo = a.offsets[g];
     const int64_t hi = (g < a.G) ? (int64_t)a.offsets[g + 1] : lo + a.extra_rows;
     if (m >= lo && m < hi) {
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
   float amax = 0.0f;
 #pragma unroll
   for (int i = 0; i < PMAX; ++i) {
-    const int n = threadIdx.x + i * 256;
+    const int n = threadIdx.x + i * NTH;
     y[i] = 0.0f;
     if (n < I) {
       if (a.acc_dbg) {
@@ -318,13 +319,15 @@ __global__ __launch_bounds__(256) void swiglu_quant_rows(GemmArgs a, int8_t* __r
   amax = wave_allmax_f(amax);
   if ((threadIdx.x & (WAVE - 1)) == 0) red[threadIdx.x / WAVE] = amax;
   __syncthreads();
-  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  amax = red[0];
+#pragma unroll
+  for (int i = 1; i < NTH / WAVE; ++i) amax = fmaxf(amax, red[i]);
   const float sc = amax / 127.0f;
   if (threadIdx.x == 0) hs[m] = sc;
   int8_t* qr = hq + (size_t)m * I;
 #pragma unroll
   for (int i = 0; i < PMAX; ++i) {
-    const int n = threadIdx.x + i * 256;
+    const int n = threadIdx.x + i * NTH;
     if (n < I) qr[n] = (sc > 0.0f) ? (int8_t)quant_i8(y[i], sc) : (int8_t)0;
   }
 }
@@ -885,8 +888,12 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
   if (rc) return rc;
   if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
-  if (I <= 256 * 8) hipLaunchKernelGGL(swiglu_quant_rows<8>, dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
-  else hipLaunchKernelGGL(swiglu_quant_rows<16>, dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
+  // few rows (decode): more threads per row shorten the per-thread chain of exp / divide sequences
+  const int rq = env_int("OMNI_MOE_ROWQ", M_cap <= 2048 ? 512 : 256);  // measured at 576 rows: 512 threads best
+  if (I > 256 * 8) hipLaunchKernelGGL((swiglu_quant_rows<16, 256>), dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
+  else if (rq == 1024 && I <= 1024 * 2) hipLaunchKernelGGL((swiglu_quant_rows<2, 1024>), dim3((unsigned)M_cap), dim3(1024), 0, st, a, h_q, h_scale);
+  else if (rq >= 512 && I <= 512 * 4) hipLaunchKernelGGL((swiglu_quant_rows<4, 512>), dim3((unsigned)M_cap), dim3(512), 0, st, a, h_q, h_scale);
+  else hipLaunchKernelGGL((swiglu_quant_rows<8, 256>), dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
   OMNI_CHECK_LAUNCH("gemm1 row epilogue");
   return OMNI_OK;
 }
