@@ -170,6 +170,19 @@ __device__ __forceinline__ int wave_incl_scan_i(int v, int lane) {
   return v;
 }
 
+// inclusive prefix sum over the 64 lanes with data-parallel-primitive moves only: shifts by 1, 2, 4, 8
+// inside each row of 16 lanes (lanes without a source add 0), then the last lane of row 0 / row 2 is
+// added to rows 1 / 3, then lane 31 to rows 2 and 3
+__device__ __forceinline__ int wave_incl_scan_dpp_i(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // floats to unsigned keys with the same order
 __device__ __forceinline__ uint32_t f32_order_key(float f) {
   uint32_t u = __float_as_uint(f);
@@ -197,6 +210,28 @@ __device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offse
                                                int b, RowBlock& rb) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int Gt = G + (extra_rows > 0 ? 1 : 0);
+  if (Gt <= WAVE) {
+    // one group per lane: everything the answer needs stays in registers after one round of loads
+    int start = 0, c = 0;
+    if (lane < Gt) {
+      start = offsets[lane < G ? lane : G];
+      c = (lane < G) ? (offsets[lane + 1] - start) : extra_rows;
+    }
+    const int nb = (c + BM - 1) / BM;
+    const int incl = wave_incl_scan_dpp_i(nb);
+    const int excl = incl - nb;
+    const int total = __builtin_amdgcn_readlane(incl, WAVE - 1);
+    if (b >= total) return false;
+    const uint64_t owner_mask = __ballot(b >= excl && b < incl);
+    const int owner = __ffsll((unsigned long long)owner_mask) - 1;
+    const int o_start = __builtin_amdgcn_readlane(start, owner);
+    const int o_c = __builtin_amdgcn_readlane(c, owner);
+    const int o_excl = __builtin_amdgcn_readlane(excl, owner);
+    rb.group = owner;
+    rb.row0 = o_start + (b - o_excl) * BM;
+    rb.nrows = min(BM, o_c - (b - o_excl) * BM);
+    return true;
+  }
   const int per = (Gt + WAVE - 1) / WAVE;
   const int g0 = lane * per;
   int mine = 0;
@@ -207,9 +242,9 @@ __device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offse
       mine += (c + BM - 1) / BM;
     }
   }
-  int incl = wave_incl_scan_i(mine, lane);
+  int incl = wave_incl_scan_dpp_i(mine);
   int excl = incl - mine;
-  int total = __shfl(incl, WAVE - 1, WAVE);
+  int total = __builtin_amdgcn_readlane(incl, WAVE - 1);
   if (b >= total) return false;
   uint64_t owner_mask = __ballot(b >= excl && b < incl);
   int owner = __ffsll((unsigned long long)owner_mask) - 1;
@@ -231,8 +266,8 @@ __device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offse
       acc += nb;
     }
   }
-  rb.group = __shfl(grp, owner, WAVE);
-  rb.row0 = __shfl(row0, owner, WAVE);
-  rb.nrows = __shfl(nrows, owner, WAVE);
+  rb.group = __builtin_amdgcn_readlane(grp, owner);
+  rb.row0 = __builtin_amdgcn_readlane(row0, owner);
+  rb.nrows = __builtin_amdgcn_readlane(nrows, owner);
   return true;
 }
