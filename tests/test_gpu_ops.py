@@ -227,3 +227,47 @@ def test_combine_k_order_with_skip(ops):
         ref = O.moe_finalize_routing(rows.float(), skip, w, p.src_to_dst.cpu(), drop_pad_mode=mode).to(torch.bfloat16)
         out = ops.moe_combine(rows.cuda(), w.cuda(), p.src_to_dst, omode, L.OMNI_ORDER_K, init=skip.cuda())
         _eq(out, ref, f"finalize mode {mode}")
+
+
+# ------------------------------------------------------------------ layer entry: extreme routings and sizes
+@pytest.mark.parametrize("T,K,n_local,E,pattern", [
+    (200, 1, 1, 4, "first_k"),    # every token to the single local expert: 200 rows in one group (tile kernel)
+    (129, 2, 4, 4, "first_k"),    # 129 rows in two groups: first size past the stream/tile switch; two empty groups
+    (128, 2, 4, 4, "first_k"),    # 128 rows: last size of the stream kernel, 4 or 8 row blocks per group
+    (257, 1, 2, 2, "first_k"),    # one row past a whole 256-row tile, one empty group
+    (40, 4, 4, 8, "none"),        # no assignment is local: only the shared expert contributes
+    (1, 8, 8, 8, "first_k"),      # one token to every expert: eight one-row groups
+    (96, 3, 5, 5, "random"),      # odd group count, ragged groups
+])
+def test_layer_entry_extreme_routings(ops, T, K, n_local, E, pattern):
+    """omni_moe_w8a8_layer (sort, both GEMMs, combine, shared expert) on routings that stress the row-block
+    logic: every token on the same experts, empty groups, nothing local, boundary row counts."""
+    H, I = 512, 256
+    g = gen(900 + T)
+    lay = Layer(n_local, H, I, seed=900 + T, shared=True)
+    x = tokens(T, H, 901 + T)
+    w = torch.rand(T, K, generator=g)
+    if pattern == "first_k":
+        ids = torch.arange(K, dtype=torch.int32).repeat(T, 1)
+    elif pattern == "none":
+        ids = torch.stack([torch.randperm(E - n_local, generator=g)[:K] + n_local for _ in range(T)]).to(torch.int32)
+    else:
+        ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    xq, xs = O.dynamic_quant(x)
+    routed = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (0, n_local))
+    shared = O.shared_expert_mlp(x, *lay.shared)
+    want = (routed.float() + shared.float()).to(torch.bfloat16)
+    d = lay.to_device()
+    out = ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), 0, n_local, d["w13"], d["s13"], d["w2"], d["s2"],
+                             (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]), H=H, I=I)
+    _eq(out, want, f"layer output ({pattern})")
+
+
+def test_layer_entry_zero_tokens(ops):
+    lay = Layer(2, 512, 256, seed=3, shared=True)
+    d = lay.to_device()
+    x = torch.zeros(0, 512, dtype=torch.bfloat16).cuda()
+    out = ops.moe_w8a8_layer(x, None, torch.zeros(0, 2).cuda(), torch.zeros(0, 2, dtype=torch.int32).cuda(), 0, 2,
+                             d["w13"], d["s13"], d["w2"], d["s2"], (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]),
+                             H=512, I=256)
+    assert out.shape == (0, 512)
