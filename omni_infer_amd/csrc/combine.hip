@@ -91,19 +91,27 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
     }
   }
   __syncthreads();
-  const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
-  if (c >= a.H) return;
+  // a block walks the column chunks blockIdx.y, blockIdx.y + gridDim.y, ... of its token
+  for (int c = (blockIdx.y * 256 + threadIdx.x) * 4; c < a.H; c += gridDim.y * 1024) {
   const int ncol = min(4, a.H - c);
   float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   if (a.init) load4<OMNI_DT_BF16>(a.init, (size_t)n, a.H, c, ncol, acc);
-  for (int j = 0; j < cnt; ++j) {
-    float v[4];
-    load4<DT, true>(a.rows, (size_t)s_slot[j], a.H, c, ncol, v);
-    const float wv = s_w[j];
+  // eight rows are requested together, then added in list order (one multiply, one add per row)
+  for (int j0 = 0; j0 < cnt; j0 += 8) {
+    float v[8][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float prod = wv * v[i];
-      acc[i] = acc[i] + prod;
+    for (int u = 0; u < 8; ++u)
+      if (j0 + u < cnt) load4<DT, true>(a.rows, (size_t)s_slot[j0 + u], a.H, c, ncol, v[u]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (j0 + u < cnt) {
+        const float wv = s_w[j0 + u];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float prod = wv * v[u][i];
+          acc[i] = acc[i] + prod;
+        }
+      }
     }
   }
   uint16_t o[4];
@@ -122,6 +130,7 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
     *(v2i*)op = t;
   } else {
     for (int j = 0; j < ncol; ++j) op[j] = o[j];
+  }
   }
 }
 
@@ -142,7 +151,10 @@ extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* t
     OMNI_FAIL(OMNI_E_INVALID, "combine: misaligned pointer");
   CombineArgs a{rows, rows_dtype, topk_w, src_to_dst, idx_mode, order, T, K, H, (const uint16_t*)init_bf16, post_add,
                 post_add_row0, (uint16_t*)out_bf16};
-  dim3 grid((unsigned)T, (unsigned)((H + 1023) / 1024)), block(256);
+  // few tokens: one block per (token, 1024-column chunk) for parallelism; many tokens: one block per
+  // token walks all chunks, so that a row's bytes are requested close together in time
+  const unsigned chunks = (unsigned)((H + 1023) / 1024);
+  dim3 grid((unsigned)T, T >= 2048 ? 1u : chunks), block(256);
   hipStream_t st = (hipStream_t)stream;
   if (rows_dtype == OMNI_DT_F32) hipLaunchKernelGGL(combine_kernel<OMNI_DT_F32>, grid, block, 0, st, a);
   else hipLaunchKernelGGL(combine_kernel<OMNI_DT_BF16>, grid, block, 0, st, a);
