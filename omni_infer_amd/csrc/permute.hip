@@ -161,10 +161,16 @@ __global__ __launch_bounds__(256) void permute_scan(PermArgs a) {
   const int nb = a.G + 1;
   for (int b = threadIdx.x; b < nb; b += 256) {
     int run = 0;
-    for (int k = 0; k < a.nblk; ++k) {
-      int c = a.blk_hist[(size_t)k * NB + b];
-      a.blk_hist[(size_t)k * NB + b] = run;
-      run += c;
+    // eight blocks' counts are requested together before their prefixes are written back
+    for (int k0 = 0; k0 < a.nblk; k0 += 8) {
+      int c[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) c[u] = (k0 + u < a.nblk) ? a.blk_hist[(size_t)(k0 + u) * NB + b] : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (k0 + u < a.nblk) a.blk_hist[(size_t)(k0 + u) * NB + b] = run;
+        run += c[u];
+      }
     }
     tot[b] = run;
   }
