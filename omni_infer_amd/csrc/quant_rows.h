@@ -47,7 +47,7 @@ __device__ __forceinline__ void quant_row_vec_body(const void* __restrict__ xv, 
     int vi = threadIdx.x + i * 256;
     if (vi < nvec) {
       if constexpr (sizeof(ET) == 2) {
-        v4i raw = *(const v4i*)(x + (size_t)vi * 8);
+        v4i raw = __builtin_nontemporal_load((const v4i*)(x + (size_t)vi * 8));  // the row is read once here
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           uint32_t u = (uint32_t)raw[j];
@@ -55,8 +55,8 @@ __device__ __forceinline__ void quant_row_vec_body(const void* __restrict__ xv, 
           v[i][2 * j + 1] = Elem<DT>::cvt((uint16_t)(u >> 16));
         }
       } else {
-        v4f a = *(const v4f*)(x + (size_t)vi * 8);
-        v4f b = *(const v4f*)(x + (size_t)vi * 8 + 4);
+        v4f a = __builtin_nontemporal_load((const v4f*)(x + (size_t)vi * 8));
+        v4f b = __builtin_nontemporal_load((const v4f*)(x + (size_t)vi * 8 + 4));
 #pragma unroll
         for (int j = 0; j < 4; ++j) { v[i][j] = a[j]; v[i][4 + j] = b[j]; }
       }
