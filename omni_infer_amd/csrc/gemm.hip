@@ -48,6 +48,7 @@ struct GemmArgs {
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
   int32_t* acc_dbg;    // [M_cap, N], nullable
+  int tile_gx, tile_gy, tile_pc;  // tile kernel: column tiles, row blocks (worst case), columns of a patch
   int32_t* part;       // GEMM1 stream kernel: [S, M_cap, N] partial accumulators (split-k)
   int S;               // number of k splits (grid.z)
   int64_t M_cap;
@@ -438,8 +439,23 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   c.wm = c.w / WN;
   c.wn = c.w % WN;
   const int lane = c.lane, w = c.w, wm = c.wm, wn = c.wn;
+  // Workgroups go to the 8 XCDs (each with its own L2) round-robin by their linear id, and about one
+  // block per CU is resident at a time.  Tile coordinates are therefore dealt so that the blocks an
+  // XCD runs together form compact patches of TILE_PR row blocks x tile_pc column tiles: the tiles
+  // of a patch share their row panels and (inside an expert) their weight panels in that L2.
+  constexpr int TILE_PR = 4;
+  int bx, by;
+  {
+    const unsigned id = blockIdx.x, xcd = id & 7u, j = id >> 3;
+    const unsigned per_patch = TILE_PR * a.tile_pc;
+    const unsigned patch = (j / per_patch) * 8u + xcd, q = j % per_patch;
+    const unsigned npc = a.tile_gx / a.tile_pc;  // patches across the columns
+    by = (int)((patch / npc) * TILE_PR + q / a.tile_pc);
+    bx = (int)((patch % npc) * a.tile_pc + q % a.tile_pc);
+    if (by >= a.tile_gy) return;
+  }
   RowBlock rb;
-  if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, blockIdx.y, rb)) return;
+  if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, by, rb)) return;
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int nk64 = a.Kdim / 64;
   const int I = (KIND == 1) ? a.N / 2 : 0;
@@ -449,8 +465,8 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // block-level strips j = 0..NBS-1: KIND 1: gate strips GS*bx.. then the matching up strips;
   // KIND 2: strips NBS*bx...  A 32-channel tile is a pair of neighbouring strips.
   auto strip_of = [&](int j) -> int {
-    if constexpr (KIND == 1) return (j < GS) ? blockIdx.x * GS + j : I / 16 + blockIdx.x * GS + (j - GS);
-    else return blockIdx.x * NBS + j;
+    if constexpr (KIND == 1) return (j < GS) ? bx * GS + j : I / 16 + bx * GS + (j - GS);
+    else return bx * NBS + j;
   };
 #pragma unroll
   for (int i = 0; i < AP; ++i) {
@@ -520,10 +536,10 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   float wsc_g[2];
   int ncol[2];
   if constexpr (KIND == 1) {
-    ncol[0] = (blockIdx.x * GS + 2 * wn) * 16 + c32;
+    ncol[0] = (bx * GS + 2 * wn) * 16 + c32;
     ncol[1] = I + ncol[0];
   } else {
-    ncol[0] = (blockIdx.x * NBS + 4 * wn) * 16 + c32;
+    ncol[0] = (bx * NBS + 4 * wn) * 16 + c32;
     ncol[1] = ncol[0] + 32;
   }
   wsc_g[0] = wsc[ncol[0]];
@@ -779,17 +795,26 @@ int tile_wn(int kind, int units) {
 }
 
 template <int KIND>
-void launch_tile(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
+void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
   const int BM = 256;
+  GemmArgs a = a0;
   const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
-  int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
-  if (tile_wn(KIND, units) == 4) {
-    dim3 grid((unsigned)(units / ((KIND == 1) ? 8 : 16)), (unsigned)mblocks), block(512);
-    if (KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE)) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1>), grid, block, 0, st, a);
+  const int wn = tile_wn(KIND, units);
+  a.tile_gx = units / ((KIND == 1) ? 2 * wn : 4 * wn);
+  a.tile_gy = (int)((M_cap + BM - 1) / BM + Gt);
+  a.tile_pc = 1;
+  for (int c = 1; c <= 8; ++c)
+    if (a.tile_gx % c == 0) a.tile_pc = c;
+  // whole patches (4 row blocks x tile_pc column tiles), dealt to the XCDs in rounds of 8
+  const int64_t patches = (int64_t)((a.tile_gy + 3) / 4) * (a.tile_gx / a.tile_pc);
+  const int64_t nblocks = (patches + 7) / 8 * 8 * 4 * a.tile_pc;
+  dim3 grid((unsigned)nblocks), block(128 * wn);
+  const bool bfi = KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE);
+  if (wn == 4) {
+    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((gemm_pipe<KIND, 4, false>), grid, block, 0, st, a);
   } else {
-    dim3 grid((unsigned)(units / ((KIND == 1) ? 4 : 8)), (unsigned)mblocks), block(256);
-    if (KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE)) hipLaunchKernelGGL((gemm_pipe<KIND, 2, KIND == 1>), grid, block, 0, st, a);
+    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 2, KIND == 1>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((gemm_pipe<KIND, 2, false>), grid, block, 0, st, a);
   }
 }
