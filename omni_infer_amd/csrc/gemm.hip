@@ -593,6 +593,8 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     for (int mt = 0; mt < 4; ++mt) {
       const int tile_r0 = wm * 128 + mt * 32;
       if (tile_r0 < nrows) {
+        float* ytile = nullptr;  // GEMM1: y element of the lane's first row of this 32-row tile
+        if constexpr (KIND == 1) ytile = a.y + (size_t)(row0 + tile_r0 + 4 * (lane >> 5)) * I + ncol[0];
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int rr = tile_r0 + tile32_row(lane, i);
@@ -606,22 +608,32 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
               if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
               float yv = silu_spec(dg) * du;
               if (bf) yv = round_bf16(yv);
-              __builtin_nontemporal_store(yv, &a.y[m * I + ncol[0]]);  // read once, by the row quantiser
-              if (a.acc_dbg) {
-                a.acc_dbg[m * (size_t)a.N + ncol[0]] = acc[mt][0][i];
-                a.acc_dbg[m * (size_t)a.N + ncol[1]] = acc[mt][1][i];
-              }
+              // entry i is row 8*(i/4) + i%4 below the lane's first row: a wave-uniform offset
+              __builtin_nontemporal_store(yv, ytile + (size_t)(8 * (i >> 2) + (i & 3)) * I);  // read once, by the row quantiser
             }
           } else if (ok) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
               float o = ((float)acc[mt][t][i] * wsc_g[t]) * ts;
               __builtin_nontemporal_store(o, &((float*)a.rows_out)[m * (size_t)a.N + ncol[t]]);
-              if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + ncol[t]] = acc[mt][t][i];
             }
           }
         }
       }
+    }
+    // raw accumulators for the parity tests, kept out of the loop above so that none of their
+    // address arithmetic is ever part of it
+    if (a.acc_dbg) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int rr = wm * 128 + mt * 32 + tile32_row(lane, i);
+          if (rr < nrows) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) a.acc_dbg[(size_t)(row0 + rr) * (size_t)a.N + ncol[t]] = acc[mt][t][i];
+          }
+        }
     }
   }
 #endif
