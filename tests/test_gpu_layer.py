@@ -217,15 +217,18 @@ def test_config3_prefill_outliers_reduced(env):
 
 
 # ------------------------------------------------------------------ config 4: Pangu-Ultra-MoE shape
-@pytest.mark.parametrize("T", [1, 16, 128])
+@pytest.mark.parametrize("T", [1, 16, 128, 1024])
 def test_config4_pangu_shape(env, T):
-    """H=7680, I=2048, 4 local experts of 32, top-8 sigmoid grouped routing, shared expert."""
+    """H=7680, I=2048, 4 local experts of 32, top-8 sigmoid grouped routing, shared expert.
+    1024 tokens put both GEMMs on the tile kernel at these widths (120 k-steps, 30 column tiles)."""
     blk, lay, gate_w, bias, lo = _dsv3_block(env, 4, 8, 1, H=7680, I=2048, seed=31)
     x = tokens(T, 7680, 31 + T)
     logits = blk.gate(x.cuda().float())[0]
     out_ref, st = _block_reference(lay, x, logits.cpu(), bias, lo, 4)
     out, _ = blk(x.cuda(), None, None, 3)
-    _check_out(out, out_ref)
+    # at 1024 tokens the fp32 row buffer would pass 256 MiB, so the rows between GEMM2 and the combine are
+    # bf16 (the numerics of the separate GEMM2 and finalize operators): tolerance instead of bit equality
+    _check_out(out, out_ref, exact=T < 1024)
 
 
 # ------------------------------------------------------------------ config 5: skewed load
