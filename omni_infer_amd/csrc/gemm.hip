@@ -758,7 +758,10 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
   int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // tuning aid: 1 stream, 2 tile
   if (force == 1) p.tile = false;
   if (force == 2) p.tile = true;
-  if (p.tile && units % ((KIND == 1) ? 4 : 8) != 0) p.tile = false;
+  const bool tile_ok = units % ((KIND == 1) ? 4 : 8) == 0;  // the tile kernel takes 64 / 128 channels at least
+  if (p.tile && !tile_ok) p.tile = false;
+  // the stream kernel walks the reduction in chunks of 256: other lengths go to the tile kernel
+  if (!p.tile && Kdim % 256 != 0 && tile_ok && force != 1) p.tile = true;
   p.mt = per <= 10 ? 1 : 2;
   p.S = 1;
   if (KIND == 1) {

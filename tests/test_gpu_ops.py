@@ -271,3 +271,48 @@ def test_layer_entry_zero_tokens(ops):
                              d["w13"], d["s13"], d["w2"], d["s2"], (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]),
                              H=512, I=256)
     assert out.shape == (0, 512)
+
+
+# ------------------------------------------------------------------ seeded sweep over small shapes
+def _sweep_cases():
+    """40 seeded shapes: token counts around the kernel-switch points, odd expert counts, all the
+    width granularities the kernels accept (reduction lengths in multiples of 256 for the stream
+    kernel, of 64 for the tile kernel), with and without the shared expert, both index modes."""
+    g = gen(4242)
+    cases = []
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for n in range(40):
+        E = r(1, 12)
+        n_local = r(1, E)
+        K = r(1, min(E, 4))
+        T = [1, 2, 7, 31, 64, 65, 130, 200, 300, 513][n % 10]
+        H = 256 * r(1, 3) if n % 3 else 64 * r(1, 9)
+        I = 256 * r(1, 2) if n % 3 else 64 * r(1, 5)
+        cases.append((T, K, n_local, E, H, I, bool(n & 1), n))
+    return cases
+
+
+@pytest.mark.parametrize("T,K,n_local,E,H,I,shared,seed", _sweep_cases())
+def test_layer_entry_shape_sweep(ops, T, K, n_local, E, H, I, shared, seed):
+    g = gen(5000 + seed)
+    lay = Layer(n_local, H, I, seed=5000 + seed, shared=shared)
+    x = tokens(T, H, 6000 + seed)
+    ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    w = torch.rand(T, K, generator=g)
+    lo = int(torch.randint(0, E - n_local + 1, (1,), generator=g))     # the local range anywhere in [0, E)
+    xq, xs = O.dynamic_quant(x)
+    routed = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (lo, lo + n_local))
+    want = routed
+    if shared:
+        want = (routed.float() + O.shared_expert_mlp(x, *lay.shared).float()).to(torch.bfloat16)
+    d = lay.to_device()
+    sh = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]) if shared else None
+    try:
+        out = ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), lo, lo + n_local, d["w13"], d["s13"], d["w2"],
+                                 d["s2"], sh, H=H, I=I)
+    except RuntimeError as e:
+        # the only widths refused: GEMM2 can use neither kernel (stream: I % 256 == 0; tile: H % 128 == 0)
+        assert I % 256 != 0 and H % 128 != 0, f"refused a supported shape: {e}"
+        assert "multiple of 256" in str(e) or "not divisible" in str(e), str(e)
+        return
+    _eq(out, want, f"layer output T={T} K={K} n_local={n_local}/{E} H={H} I={I} shared={shared}")
