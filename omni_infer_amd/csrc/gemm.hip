@@ -476,11 +476,15 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) c.bsrc[i] = wbase + (size_t)strip_of(2 * w + i) * nk64 * 1024 + lane * 16;
-  // per-row activation scales go to LDS once (read back in the epilogue)
+  // the first two k-steps are requested as soon as their addresses exist; everything else the block
+  // has to set up overlaps with their flight
+  const int last = nk64 - 1;
+  pipe_load<WN>(c, 0, sa0, sb0);
+  pipe_load<WN>(c, min(1, last), sa1, sb1);
+  // per-row activation scales go to LDS once (read back in the epilogue, after many barriers)
   for (int r = threadIdx.x; r < BM; r += 128 * WN) {
     row_scale[r] = (r < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + r)] : 0.0f;
   }
-  __syncthreads();
   // operand addressing of the 32x32x32 form (see the header comment)
   const int in_pair = ((lane & 31) >> 4) * WAVE + (lane & 15) + 16 * (lane >> 5);
   c.a_off = (wm * 8) * WAVE + in_pair;
@@ -500,9 +504,6 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
 
-  const int last = nk64 - 1;
-  pipe_load<WN>(c, 0, sa0, sb0);
-  pipe_load<WN>(c, min(1, last), sa1, sb1);
   int ks = 0;
   for (; ks + 3 <= nk64; ks += 3) {
     pipe_sync<WN>();
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   constexpr int OUT_PITCH_DW = 48;
   const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
   uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * (32 * OUT_PITCH_DW);
-  if (bf16_out) __syncthreads();  // every wavefront is done reading the last stage
+  __syncthreads();  // every wavefront is done reading the last stage; the row scales written at the start are visible
   constexpr bool bf = BF;
   float wsc_g[2];
   int ncol[2];
