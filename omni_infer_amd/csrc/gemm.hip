@@ -140,6 +140,15 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
 #pragma unroll
   for (int j = 0; j < NBF; ++j) bp[j] = wbase + ((size_t)strip[j] * nk64_all + k64_0) * 1024 + lane * 16;
 
+  // the first D k-steps of B are requested as soon as their addresses exist (they come from HBM and
+  // take the longest); the A row lookup below overlaps with their flight
+  v4i ring[D][NBF];
+#pragma unroll
+  for (int s = 0; s < D; ++s)
+#pragma unroll
+    for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
+  __builtin_amdgcn_sched_barrier(0);
+
   // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile, k-step w of
   // every chunk; rows past the end of the group alias the group's first row
   const int8_t* arow[MT];
@@ -156,15 +165,10 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
 #pragma unroll
     for (int j = 0; j < NBF; ++j) acc[mt][j] = (v4i){0, 0, 0, 0};
 
-  // ---- prologue: A chunk 0 -> LDS, first D k-steps of B -> ring
+  // ---- prologue: A chunk 0 -> LDS
   v4i areg[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt]);
-  v4i ring[D][NBF];
-#pragma unroll
-  for (int s = 0; s < D; ++s)
-#pragma unroll
-    for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) lds_a[0][(mt * 4 + w) * WAVE + lane] = areg[mt];
   __syncthreads();
