@@ -302,3 +302,54 @@ def test_full_size_properties(env, T):
     e1 = run(x, w, ids, None)
     e2 = run(x, w * 2, ids, None)
     assert torch.equal(e2.float(), e1.float() * 2), "routing weights are not applied linearly"
+
+
+# ------------------------------------------------------------------ HIP graph capture of the call sequence
+def test_layer_call_sequence_is_graph_capturable(env):
+    """Router + whole-layer entry captured in a HIP graph (no allocation, synchronisation or host read
+    inside the library), replayed three times with eager work and synchronisations in between; every
+    replay must give the bits of the eager run, also after the inputs changed in place."""
+    T, K, E, n, H, I = 64, 8, 32, 4, 1024, 512
+    lay = Layer(n, H, I, seed=77, shared=True)
+    d = lay.to_device()
+    g = gen(78)
+    x = tokens(T, H, 79).cuda()
+    logits = torch.randn(T, E, generator=g).cuda()
+    bias = (torch.randn(E, generator=g) * 0.01).cuda()
+    ops, L = env.ops, env.L
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n, H, I, 1)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out = torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+
+    def step():
+        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, 4, 8, 1, 0, 1, 2.5, 1e-20)
+        return ops.moe_w8a8_layer(x, None, w, ids, 0, n, d["w13"], d["s13"], d["w2"], d["s2"], shared, H=H, I=I,
+                                  workspace=ws, out=out)
+
+    eager = step().clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                               # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        out.zero_()
+        junk = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")   # eager work in between
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager run"
+        del junk
+    # new inputs in the captured buffers
+    x.copy_(tokens(T, H, 80).cuda())
+    logits.copy_(torch.randn(T, E, generator=g).cuda())
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = out.clone()
+    assert torch.equal(step(), replayed), "replay on new inputs differs from the eager run"
