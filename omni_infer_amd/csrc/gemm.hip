@@ -422,6 +422,128 @@ __device__ __forceinline__ void pipe_sync() {
 // 32x32 accumulator tile: lane l holds column l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 __device__ __forceinline__ int tile32_row(int lane, int i) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }
 
+// Epilogue of one 256 x (64*WN) tile, shared by the tile kernels: a wavefront holds a 128 x 64 piece as
+// 4 x 2 accumulator tiles of 32 x 32.  GEMM1: dequantise, SwiGLU, y (fp32) with streaming stores.
+// GEMM2: fp32 rows, or bf16 rows transposed through LDS (stage32: a private 32 x 64 piece per
+// wavefront, rows padded to 192 bytes = 48 dwords, so that the two rows a half-wavefront writes at
+// once fall into disjoint banks) and stored as whole 128-byte lines.
+constexpr int TILE_OUT_PITCH_DW = 48;
+#define TILE_STAGE_DWORDS (32 * TILE_OUT_PITCH_DW)  // staging dwords of one wavefront
+template <int KIND, int WN, bool BF>
+__device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][2], const float* row_scale,
+                                              uint32_t* stage32, int lane, int wm, int wn, int bx, int row0,
+                                              int nrows, const float* __restrict__ wsc, int I) {
+  constexpr int NBS = 4 * WN;
+  constexpr int GS = 2 * WN;
+  // ---- epilogue, one 32-row tile at a time
+  const int c32 = lane & 31;
+  constexpr int OUT_PITCH_DW = TILE_OUT_PITCH_DW;
+  const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
+  constexpr bool bf = BF;
+  float wsc_g[2];
+  int ncol[2];
+  if constexpr (KIND == 1) {
+    ncol[0] = (bx * GS + 2 * wn) * 16 + c32;
+    ncol[1] = I + ncol[0];
+  } else {
+    ncol[0] = (bx * NBS + 4 * wn) * 16 + c32;
+    ncol[1] = ncol[0] + 32;
+  }
+  wsc_g[0] = wsc[ncol[0]];
+  wsc_g[1] = wsc[ncol[1]];
+  if (bf16_out) {
+    if constexpr (KIND == 2) {
+      const int odd = c32 & 1;
+      // byte selector of v_perm_b32 over {theirs (bytes 4-7), mine (bytes 0-3)}: even lanes keep
+      // their low half and take the neighbour's low half on top, odd lanes take the neighbour's
+      // high half below their own high half
+      const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
+      uint32_t* const stage_lane = stage32 + (4 * (lane >> 5) + odd) * OUT_PITCH_DW + (c32 >> 1);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        const int tile_r0 = wm * 128 + mt * 32;
+        if (tile_r0 < nrows) {
+          // accumulator entries i, i+1 (i even) are rows r, r+1 of the same channel; neighbouring
+          // lanes hold neighbouring channels.  One pack, one lane exchange and one byte permute give
+          // every lane a dword of two neighbouring channels: even lanes for row r, odd lanes for row r+1.
+          const float* ts_lane = row_scale + tile_r0 + 4 * (lane >> 5);
+#pragma unroll
+          for (int i = 0; i < 16; i += 2) {
+            const int rr = 8 * (i >> 2) + (i & 3);  // row below the lane's first row of the tile
+            const float ts0 = ts_lane[rr], ts1 = ts_lane[rr + 1];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              const float o0 = ((float)acc[mt][t][i] * wsc_g[t]) * ts0;
+              const float o1 = ((float)acc[mt][t][i + 1] * wsc_g[t]) * ts1;
+              const uint32_t mine = f32x2_to_bf16x2(o0, o1);
+              const uint32_t theirs = (uint32_t)xchg_i<1>((int)mine);
+              stage_lane[rr * OUT_PITCH_DW + t * 16] = __builtin_amdgcn_perm(theirs, mine, sel);
+            }
+          }
+          // the wavefront wrote its 32 x 64 piece; now 8 lanes per row store 16 bytes each
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = j * 8 + (lane >> 3);
+            const int rr = tile_r0 + r;
+            v4i v = *(const v4i*)(stage32 + r * OUT_PITCH_DW + (lane & 7) * 4);
+            if (rr < nrows)  // read once, by the combine
+              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int tile_r0 = wm * 128 + mt * 32;
+      if (tile_r0 < nrows) {
+        float* ytile = nullptr;  // GEMM1: y element of the lane's first row of this 32-row tile
+        if constexpr (KIND == 1) ytile = a.y + (size_t)(row0 + tile_r0 + 4 * (lane >> 5)) * I + ncol[0];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int rr = tile_r0 + tile32_row(lane, i);
+          const bool ok = rr < nrows;
+          const size_t m = (size_t)(row0 + rr);
+          const float ts = row_scale[rr];
+          if constexpr (KIND == 1) {
+            if (ok) {
+              float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
+              float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
+              if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+              float yv = silu_spec(dg) * du;
+              if (bf) yv = round_bf16(yv);
+              // entry i is row 8*(i/4) + i%4 below the lane's first row: a wave-uniform offset
+              __builtin_nontemporal_store(yv, ytile + (size_t)(8 * (i >> 2) + (i & 3)) * I);  // read once, by the row quantiser
+            }
+          } else if (ok) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+              float o = ((float)acc[mt][t][i] * wsc_g[t]) * ts;
+              __builtin_nontemporal_store(o, &((float*)a.rows_out)[m * (size_t)a.N + ncol[t]]);
+            }
+          }
+        }
+      }
+    }
+  }
+  // raw accumulators for the parity tests, kept out of the loops above so that none of their
+  // address arithmetic is ever part of them
+  if (a.acc_dbg) {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int rr = wm * 128 + mt * 32 + tile32_row(lane, i);
+        if (rr < nrows) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) a.acc_dbg[(size_t)(row0 + rr) * (size_t)a.N + ncol[t]] = acc[mt][t][i];
+        }
+      }
+  }
+}
+
 // WN = 2: 256 threads, tile 256 x 128, two blocks per CU.  WN = 4: 512 threads, tile 256 x 256, one block
 // per CU (a third fewer operand bytes through the vector memory path per MFMA).
 // BF (GEMM1 only): round gate, up and their product to bf16 (the numerics of the reference's
@@ -528,119 +650,11 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // no LDS traffic may still be in flight when the block's LDS is handed to the next block
   __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));  // vmcnt(0)
 
-  // ---- epilogue, one 32-row tile at a time
-  const int c32 = lane & 31;
-  // bf16 rows of GEMM2 are transposed through LDS (the stage buffers are free now): a private
-  // 32 x 64 piece per wavefront, rows padded to 192 bytes (48 dwords: the two rows a half-wavefront
-  // writes at once then fall into disjoint banks); two wavefronts share a stage buffer
-  constexpr int OUT_PITCH_DW = 48;
-  const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
-  uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * (32 * OUT_PITCH_DW);
+  // ---- epilogue (the stage buffers are free now: the bf16 rows of GEMM2 are staged there, two
+  // wavefronts per buffer)
   __syncthreads();  // every wavefront is done reading the last stage; the row scales written at the start are visible
-  constexpr bool bf = BF;
-  float wsc_g[2];
-  int ncol[2];
-  if constexpr (KIND == 1) {
-    ncol[0] = (bx * GS + 2 * wn) * 16 + c32;
-    ncol[1] = I + ncol[0];
-  } else {
-    ncol[0] = (bx * NBS + 4 * wn) * 16 + c32;
-    ncol[1] = ncol[0] + 32;
-  }
-  wsc_g[0] = wsc[ncol[0]];
-  wsc_g[1] = wsc[ncol[1]];
-  if (bf16_out) {
-    if constexpr (KIND == 2) {
-      const int odd = c32 & 1;
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        const int tile_r0 = wm * 128 + mt * 32;
-        if (tile_r0 < nrows) {
-          // accumulator entries i, i+1 (i even) are rows r, r+1 of the same channel; neighbouring
-          // lanes hold neighbouring channels.  One pack + one lane exchange gives every lane a
-          // dword of two neighbouring channels: even lanes for row r, odd lanes for row r+1.
-#pragma unroll
-          for (int i = 0; i < 16; i += 2) {
-            const int r = tile32_row(lane, i);
-            const float ts0 = row_scale[tile_r0 + r], ts1 = row_scale[tile_r0 + r + 1];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-              const float o0 = ((float)acc[mt][t][i] * wsc_g[t]) * ts0;
-              const float o1 = ((float)acc[mt][t][i + 1] * wsc_g[t]) * ts1;
-              const uint32_t mine = f32x2_to_bf16x2(o0, o1);
-              const uint32_t theirs = (uint32_t)xchg_i<1>((int)mine);
-              const uint32_t out = odd ? ((theirs >> 16) | (mine & 0xffff0000u)) : ((mine & 0xffffu) | (theirs << 16));
-              stage32[(r + odd) * OUT_PITCH_DW + t * 16 + (c32 >> 1)] = out;
-              if (a.acc_dbg) {
-#pragma unroll
-                for (int d = 0; d < 2; ++d)
-                  if (tile_r0 + r + d < nrows)
-                    a.acc_dbg[(size_t)(row0 + tile_r0 + r + d) * (size_t)a.N + ncol[t]] = acc[mt][t][i + d];
-              }
-            }
-          }
-          // the wavefront wrote its 32 x 64 piece; now 8 lanes per row store 16 bytes each
-          __builtin_amdgcn_wave_barrier();
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int r = j * 8 + (lane >> 3);
-            const int rr = tile_r0 + r;
-            v4i v = *(const v4i*)(stage32 + r * OUT_PITCH_DW + (lane & 7) * 4);
-            if (rr < nrows)  // read once, by the combine
-              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
-          }
-          __builtin_amdgcn_wave_barrier();
-        }
-      }
-    }
-  } else {
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      const int tile_r0 = wm * 128 + mt * 32;
-      if (tile_r0 < nrows) {
-        float* ytile = nullptr;  // GEMM1: y element of the lane's first row of this 32-row tile
-        if constexpr (KIND == 1) ytile = a.y + (size_t)(row0 + tile_r0 + 4 * (lane >> 5)) * I + ncol[0];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int rr = tile_r0 + tile32_row(lane, i);
-          const bool ok = rr < nrows;
-          const size_t m = (size_t)(row0 + rr);
-          const float ts = row_scale[rr];
-          if constexpr (KIND == 1) {
-            if (ok) {
-              float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
-              float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
-              if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
-              float yv = silu_spec(dg) * du;
-              if (bf) yv = round_bf16(yv);
-              // entry i is row 8*(i/4) + i%4 below the lane's first row: a wave-uniform offset
-              __builtin_nontemporal_store(yv, ytile + (size_t)(8 * (i >> 2) + (i & 3)) * I);  // read once, by the row quantiser
-            }
-          } else if (ok) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-              float o = ((float)acc[mt][t][i] * wsc_g[t]) * ts;
-              __builtin_nontemporal_store(o, &((float*)a.rows_out)[m * (size_t)a.N + ncol[t]]);
-            }
-          }
-        }
-      }
-    }
-    // raw accumulators for the parity tests, kept out of the loop above so that none of their
-    // address arithmetic is ever part of it
-    if (a.acc_dbg) {
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int rr = wm * 128 + mt * 32 + tile32_row(lane, i);
-          if (rr < nrows) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t) a.acc_dbg[(size_t)(row0 + rr) * (size_t)a.N + ncol[t]] = acc[mt][t][i];
-          }
-        }
-    }
-  }
+  uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
+  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wm, wn, bx, row0, nrows, wsc, I);
 #endif
 }
 
