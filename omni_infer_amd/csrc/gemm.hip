@@ -26,6 +26,7 @@
 // row into a per-row word with an atomic max on the float's bit pattern (exact and order
 // independent for non-negative floats); a second small kernel quantises the rows.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -495,37 +496,47 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
       }
     }
   } else {
+    // one 32-row tile: FULL (all 32 rows exist, the common case) carries no per-row test, so the 16
+    // entries of a lane form one straight run of independent arithmetic chains
+    auto rows32 = [&](int mt, int tile_r0, auto full) {
+      constexpr bool FULL = decltype(full)::value;
+      // the lane's 16 rows are 4 runs of 4 consecutive rows: their scales come as 4 vector reads
+      const v4f* ts4 = (const v4f*)(row_scale + tile_r0 + 4 * (lane >> 5));
+      v4f ts[4];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      const int tile_r0 = wm * 128 + mt * 32;
-      if (tile_r0 < nrows) {
-        float* ytile = nullptr;  // GEMM1: y element of the lane's first row of this 32-row tile
-        if constexpr (KIND == 1) ytile = a.y + (size_t)(row0 + tile_r0 + 4 * (lane >> 5)) * I + ncol[0];
+      for (int q = 0; q < 4; ++q) ts[q] = ts4[2 * q];
+      const int lane_r0 = tile_r0 + 4 * (lane >> 5);  // the lane's first row of this tile
+      float* ytile = nullptr;    // GEMM1: y element of the lane's first row
+      float* otile = nullptr;    // GEMM2: fp32 output row element of the lane's first row, first tile
+      if constexpr (KIND == 1) ytile = a.y + (size_t)(row0 + lane_r0) * I + ncol[0];
+      else otile = (float*)a.rows_out + (size_t)(row0 + lane_r0) * (size_t)a.N + ncol[0];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int rr = tile_r0 + tile32_row(lane, i);
-          const bool ok = rr < nrows;
-          const size_t m = (size_t)(row0 + rr);
-          const float ts = row_scale[rr];
+      for (int i = 0; i < 16; ++i) {
+        const int below = 8 * (i >> 2) + (i & 3);  // entry i is this many rows below the lane's first row
+        if (FULL || lane_r0 + below < nrows) {
+          const float tsv = ts[i >> 2][i & 3];
           if constexpr (KIND == 1) {
-            if (ok) {
-              float dg = ((float)acc[mt][0][i] * wsc_g[0]) * ts;
-              float du = ((float)acc[mt][1][i] * wsc_g[1]) * ts;
-              if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
-              float yv = silu_spec(dg) * du;
-              if (bf) yv = round_bf16(yv);
-              // entry i is row 8*(i/4) + i%4 below the lane's first row: a wave-uniform offset
-              __builtin_nontemporal_store(yv, ytile + (size_t)(8 * (i >> 2) + (i & 3)) * I);  // read once, by the row quantiser
-            }
-          } else if (ok) {
+            float dg = ((float)acc[mt][0][i] * wsc_g[0]) * tsv;
+            float du = ((float)acc[mt][1][i] * wsc_g[1]) * tsv;
+            if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+            float yv = silu_spec(dg) * du;
+            if (bf) yv = round_bf16(yv);
+            __builtin_nontemporal_store(yv, ytile + (size_t)below * I);  // read once, by the row quantiser
+          } else {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-              float o = ((float)acc[mt][t][i] * wsc_g[t]) * ts;
-              __builtin_nontemporal_store(o, &((float*)a.rows_out)[m * (size_t)a.N + ncol[t]]);
+              float o = ((float)acc[mt][t][i] * wsc_g[t]) * tsv;
+              __builtin_nontemporal_store(o, otile + (size_t)below * (size_t)a.N + 32 * t);
             }
           }
         }
       }
+    };
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int tile_r0 = wm * 128 + mt * 32;
+      if (tile_r0 + 32 <= nrows) rows32(mt, tile_r0, std::true_type{});
+      else if (tile_r0 < nrows) rows32(mt, tile_r0, std::false_type{});
     }
   }
   // raw accumulators for the parity tests, kept out of the loops above so that none of their
@@ -557,7 +568,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   constexpr int AP = PipeCtx<WN>::A_PER_WAVE;
   __shared__ v4i sa0[16 * WAVE], sa1[16 * WAVE], sa2[16 * WAVE];
   __shared__ v4i sb0[NBS * WAVE], sb1[NBS * WAVE], sb2[NBS * WAVE];
-  __shared__ float row_scale[BM];     // activation scale of every row of the block
+  __shared__ __attribute__((aligned(16))) float row_scale[BM];  // activation scale of every row of the block
 
   PipeCtx<WN> c;
   c.lane = threadIdx.x & (WAVE - 1);
