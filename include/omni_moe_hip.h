@@ -56,10 +56,11 @@ extern "C" {
 /* gemm flags */
 #define OMNI_GEMM1_BF16_INTERMEDIATE 1 /* round the dequantised gate/up and the SwiGLU product to bf16
                                           (numerics of the non-EP pipeline, compressed_tensors_moe.py:242-247) */
-#define OMNI_GEMM1_NO_PROLOGUE 2  /* do not clear the row-maximum words first (the caller did) */
-#define OMNI_GEMM1_NO_REQUANT 4   /* stop after the GEMM kernel: y and the row maxima stay in the workspace,
-                                     h_q / h_scale are not written.  With NO_PROLOGUE the call is exactly one
-                                     kernel launch, which is how the benchmark times that kernel alone. */
+#define OMNI_GEMM1_NO_PROLOGUE 2  /* accepted and ignored: no kernel runs ahead of the GEMM any more */
+#define OMNI_GEMM1_NO_REQUANT 4   /* stop after the GEMM kernel: its result (int32 accumulators or fp32 y)
+                                     stays in the workspace, h_q / h_scale are not written.  The call is then
+                                     exactly one kernel launch, which is how the benchmark times that kernel
+                                     alone. */
 /* combine: how src_to_dst is indexed */
 #define OMNI_IDX_TOKEN_MAJOR 0 /* n*K + k  (npu_moe_init_routing_v2 row_idx_type=1; finalize drop_pad_mode=2) */
 #define OMNI_IDX_K_MAJOR 1     /* k*T + n  (npu_moe_init_routing; finalize drop_pad_mode=0) */

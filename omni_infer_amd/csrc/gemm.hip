@@ -832,7 +832,7 @@ void launch_stream(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) 
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }
 
-// number of channel blocks of the large-tile GEMM1 (also the number of row-maximum words per row)
+// wavefront columns of the large tile: 4 (256 channels per block) when the channel count allows, else 2
 int tile_wn(int kind, int units) {
   const int wide = (kind == 1) ? 8 : 16;  // units per 256-channel block
   const int want = env_int("OMNI_MOE_TILE_WN", 4);
