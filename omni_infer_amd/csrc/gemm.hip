@@ -366,6 +366,7 @@ struct PipeCtx {
   const int8_t* asrc[A_PER_WAVE];
   const int8_t* bsrc[2];
   int w, lane, wm, wn;
+  int mt_count;  // 32-row tiles of this wavefront that hold rows of the block (0..4)
   int a_off;     // v4i index of this lane's A operand inside the wavefront's first 32-row pair, half 0
   int b_off[2];  // same for the two 32-channel tiles of the wavefront
 };
@@ -383,30 +384,38 @@ __device__ __forceinline__ void pipe_load(const PipeCtx<WN>& c, int k, v4i* __re
 #endif
 }
 
-template <int WN>
+// PARTIAL: the wavefront owns fewer than four 32-row tiles with rows in them (the last row block of a
+// group): it reads and multiplies only those, and a wavefront without rows only takes part in the
+// loads and the barriers.  Full wavefronts run the variant without any of the tests.
+template <int WN, bool PARTIAL>
 __device__ __forceinline__ void pipe_step(const PipeCtx<WN>& c, int kload, v4i* __restrict__ dst_a,
                                           v4i* __restrict__ dst_b, const v4i* __restrict__ src_a,
                                           const v4i* __restrict__ src_b, v16i (&acc)[4][2]) {
 #if defined(__HIP_DEVICE_COMPILE__)
   pipe_load<WN>(c, kload, dst_a, dst_b);
+  if (PARTIAL && c.mt_count == 0) return;
   // operands of both halves: the second half is requested before the first half's MFMAs are issued,
   // so its LDS latency hides behind them
   v4i bf[2][2], af[2][4];
 #pragma unroll
   for (int t = 0; t < 2; ++t) bf[0][t] = src_b[c.b_off[t]];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) af[0][mt] = src_a[c.a_off + mt * 2 * WAVE];
+  for (int mt = 0; mt < 4; ++mt)
+    if (!PARTIAL || mt < c.mt_count) af[0][mt] = src_a[c.a_off + mt * 2 * WAVE];
 #pragma unroll
   for (int t = 0; t < 2; ++t) bf[1][t] = src_b[c.b_off[t] + 32];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) af[1][mt] = src_a[c.a_off + mt * 2 * WAVE + 32];
+  for (int mt = 0; mt < 4; ++mt)
+    if (!PARTIAL || mt < c.mt_count) af[1][mt] = src_a[c.a_off + mt * 2 * WAVE + 32];
 #pragma unroll
   for (int half = 0; half < 2; ++half)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
+      if (!PARTIAL || mt < c.mt_count) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-        acc[mt][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[half][mt], bf[half][t], acc[mt][t], 0, 0, 0);
+        for (int t = 0; t < 2; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[half][mt], bf[half][t], acc[mt][t], 0, 0, 0);
+      }
 #endif
 }
 
@@ -418,6 +427,32 @@ __device__ __forceinline__ void pipe_sync() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));  // vmcnt(N), other counters untouched
   __builtin_amdgcn_s_barrier();
 #endif
+}
+
+// the k loop of one tile: a ring of three stages, two k-steps in flight while one is multiplied; the first
+// two k-steps are already on their way into stages 0 and 1
+template <int WN, bool PARTIAL>
+__device__ __forceinline__ void pipe_k_loop(const PipeCtx<WN>& c, int nk64, v4i* __restrict__ sa0, v4i* __restrict__ sa1,
+                                            v4i* __restrict__ sa2, v4i* __restrict__ sb0, v4i* __restrict__ sb1,
+                                            v4i* __restrict__ sb2, v16i (&acc)[4][2]) {
+  const int last = nk64 - 1;
+  int ks = 0;
+  for (; ks + 3 <= nk64; ks += 3) {
+    pipe_sync<WN>();
+    pipe_step<WN, PARTIAL>(c, min(ks + 2, last), sa2, sb2, sa0, sb0, acc);
+    pipe_sync<WN>();
+    pipe_step<WN, PARTIAL>(c, min(ks + 3, last), sa0, sb0, sa1, sb1, acc);
+    pipe_sync<WN>();
+    pipe_step<WN, PARTIAL>(c, min(ks + 4, last), sa1, sb1, sa2, sb2, acc);
+  }
+  if (ks < nk64) {  // one or two k-steps left; the ring is back at stage 0
+    pipe_sync<WN>();
+    pipe_step<WN, PARTIAL>(c, last, sa2, sb2, sa0, sb0, acc);
+    if (ks + 1 < nk64) {
+      pipe_sync<WN>();
+      pipe_step<WN, PARTIAL>(c, last, sa0, sb0, sa1, sb1, acc);
+    }
+  }
 }
 
 // 32x32 accumulator tile: lane l holds column l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
@@ -641,23 +676,10 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
 
-  int ks = 0;
-  for (; ks + 3 <= nk64; ks += 3) {
-    pipe_sync<WN>();
-    pipe_step<WN>(c, min(ks + 2, last), sa2, sb2, sa0, sb0, acc);
-    pipe_sync<WN>();
-    pipe_step<WN>(c, min(ks + 3, last), sa0, sb0, sa1, sb1, acc);
-    pipe_sync<WN>();
-    pipe_step<WN>(c, min(ks + 4, last), sa1, sb1, sa2, sb2, acc);
-  }
-  if (ks < nk64) {  // one or two k-steps left; the ring is back at stage 0
-    pipe_sync<WN>();
-    pipe_step<WN>(c, last, sa2, sb2, sa0, sb0, acc);
-    if (ks + 1 < nk64) {
-      pipe_sync<WN>();
-      pipe_step<WN>(c, last, sa0, sb0, sa1, sb1, acc);
-    }
-  }
+  // wavefronts whose 128 rows all exist take the loop without tests
+  c.mt_count = min(4, max(0, (nrows - wm * 128 + 31) / 32));
+  if (c.mt_count == 4) pipe_k_loop<WN, false>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
+  else pipe_k_loop<WN, true>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
   // no LDS traffic may still be in flight when the block's LDS is handed to the next block
   __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));  // vmcnt(0)
 
