@@ -801,12 +801,17 @@ int env_int(const char* name, int dflt) {
 template <int KIND>
 Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_cap) {
   const int units = (KIND == 1) ? N / 32 : N / 16;  // KIND 1: (gate, up) strip pairs; KIND 2: strips
-  int64_t per = (G > 0) ? ((int64_t)T * K + G - 1) / G : 0;
-  if (per > (int64_t)T) per = T;
-  if (extra_rows > per) per = extra_rows;
+  // expected rows of a routed group (uniform routing); the shared group, when there is one, has T rows
+  int64_t avg = (G > 0) ? ((int64_t)T * K + G - 1) / G : 0;
+  if (avg > (int64_t)T) avg = T;
+  const int64_t per = (G > 0) ? avg : extra_rows;
   Plan p{};
   p.per = per;
-  p.tile = per > 128;
+  // Measured on the DeepSeek-V3 shape (32 routed groups + the shared one): up to 48 expected rows per
+  // routed group the stream kernel wins (row blocks of 64 rows from 25 expected rows on, so that
+  // nearly every group is one block and its weights are read once; the shared group then takes a few
+  // blocks and re-reads its 3 % of the bytes); above that the tile kernel does.
+  p.tile = (G > 0) ? per > 48 : per > 128;
   int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // tuning aid: 1 stream, 2 tile
   if (force == 1) p.tile = false;
   if (force == 2) p.tile = true;
@@ -814,7 +819,7 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
   if (p.tile && !tile_ok) p.tile = false;
   // the stream kernel walks the reduction in chunks of 256: other lengths go to the tile kernel
   if (!p.tile && Kdim % 256 != 0 && tile_ok && force != 1) p.tile = true;
-  p.mt = per <= 10 ? 1 : 2;
+  p.mt = per <= 10 ? 1 : (per <= 24 ? 2 : 4);
   p.S = 1;
   if (KIND == 1) {
     p.nt = 1; p.d = 4;
