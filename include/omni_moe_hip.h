@@ -183,11 +183,14 @@ size_t omni_moe_gemm1_workspace_bytes(int T, int K, int G, int extra_rows, int64
  * and npu_quant_matmul(pertoken_scale=) (schemes/compressed_tensors_w8a8_int8.py:105-109).
  *   rows_out[m, :] = cast((float(h_q[m] . W2[g]) * w2_scale[g][:]) * h_scale[m]), out_dtype BF16 or F32.
  *   w2 packed: G matrices of Kdim = I, N = H.  Grouping as in GEMM1.
+ *   workspace (omni_moe_gemm2_workspace_bytes, 256-byte aligned) is scratch for tiles whose reduction is
+ *   shared between blocks; NULL is accepted (such tiles then run unsplit, the results are the same).
  */
 int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
                            const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows,
                            const int32_t* offsets, int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out,
-                           int32_t* acc_dbg, void* stream);
+                           int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream);
+size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int H, int I);
 
 /*
  * Weighted un-permute.  Replaces the routing half of npu_grouped_matmul_finalize_routing

@@ -134,7 +134,6 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
   }
 }
 
-inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
 }  // namespace
 
@@ -191,6 +190,8 @@ LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
   L.h_q = take((size_t)L.M_cap * I);
   L.h_s = take((size_t)L.M_cap * 4);
   L.g1_bytes = omni_moe_gemm1_workspace_bytes(T, K, G, with_shared ? T : 0, L.M_cap, H, I);
+  const size_t g2_bytes = omni_moe_gemm2_workspace_bytes(G, with_shared ? T : 0, L.M_cap, H, I);
+  if (g2_bytes > L.g1_bytes) L.g1_bytes = g2_bytes;
   L.g1_ws = take(L.g1_bytes);
   L.rows_dtype = ((size_t)L.M_cap * H * 4 <= ROWS_F32_LIMIT) ? OMNI_DT_F32 : OMNI_DT_BF16;
   L.rows = take((size_t)L.M_cap * H * (L.rows_dtype == OMNI_DT_F32 ? 4 : 2));
@@ -254,8 +255,10 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
                                    sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),
                                    (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, stream);
   if (rc) return rc;
+  // GEMM1's scratch is free again once its row quantiser has run: GEMM2 takes it over
   rc = omni_moe_gemm2_dequant((const int8_t*)(ws + L.h_q), (const float*)(ws + L.h_s), w2_packed, w2_scale, sh2_packed,
-                              sh2_scale, extra, offsets, G, H, I, L.M_cap, L.rows_dtype, ws + L.rows, nullptr, stream);
+                              sh2_scale, extra, offsets, G, H, I, L.M_cap, L.rows_dtype, ws + L.rows, nullptr,
+                              ws + L.g1_ws, L.g1_bytes, stream);
   if (rc) return rc;
   return omni_moe_combine(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
                           nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,

@@ -16,6 +16,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 #define WAVE 64
 
+inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
 // ---------------------------------------------------------------- host side error state
 void omni_set_error(const char* fmt, ...);
 #define OMNI_FAIL(code, ...)        \
@@ -206,31 +208,28 @@ struct RowBlock {
   int row0;
   int nrows;
 };
-__device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offsets, int G, int extra_rows, int BM,
-                                               int b, RowBlock& rb) {
+// Row blocks of BM rows, group by group (the extra group last).  The scan is done once per
+// wavefront (every lane takes part); any number of lookups can follow.
+struct RowBlockScan {
+  int start, c, incl, nb;  // Gt <= 64: this lane's group (first row, rows, inclusive block prefix, blocks)
+  int total;               // row blocks over all groups
+  bool small;              // one group per lane
+};
+__device__ __forceinline__ RowBlockScan row_blocks_scan(const int32_t* __restrict__ offsets, int G, int extra_rows, int BM) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int Gt = G + (extra_rows > 0 ? 1 : 0);
-  if (Gt <= WAVE) {
-    // one group per lane: everything the answer needs stays in registers after one round of loads
-    int start = 0, c = 0;
+  RowBlockScan s{};
+  s.small = Gt <= WAVE;
+  if (s.small) {
+    // one group per lane: everything a lookup needs stays in registers after one round of loads
     if (lane < Gt) {
-      start = offsets[lane < G ? lane : G];
-      c = (lane < G) ? (offsets[lane + 1] - start) : extra_rows;
+      s.start = offsets[lane < G ? lane : G];
+      s.c = (lane < G) ? (offsets[lane + 1] - s.start) : extra_rows;
     }
-    const int nb = (c + BM - 1) / BM;
-    const int incl = wave_incl_scan_dpp_i(nb);
-    const int excl = incl - nb;
-    const int total = __builtin_amdgcn_readlane(incl, WAVE - 1);
-    if (b >= total) return false;
-    const uint64_t owner_mask = __ballot(b >= excl && b < incl);
-    const int owner = __ffsll((unsigned long long)owner_mask) - 1;
-    const int o_start = __builtin_amdgcn_readlane(start, owner);
-    const int o_c = __builtin_amdgcn_readlane(c, owner);
-    const int o_excl = __builtin_amdgcn_readlane(excl, owner);
-    rb.group = owner;
-    rb.row0 = o_start + (b - o_excl) * BM;
-    rb.nrows = min(BM, o_c - (b - o_excl) * BM);
-    return true;
+    s.nb = (s.c + BM - 1) / BM;
+    s.incl = wave_incl_scan_dpp_i(s.nb);
+    s.total = __builtin_amdgcn_readlane(s.incl, WAVE - 1);
+    return s;
   }
   const int per = (Gt + WAVE - 1) / WAVE;
   const int g0 = lane * per;
@@ -242,12 +241,30 @@ __device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offse
       mine += (c + BM - 1) / BM;
     }
   }
-  int incl = wave_incl_scan_dpp_i(mine);
-  int excl = incl - mine;
-  int total = __builtin_amdgcn_readlane(incl, WAVE - 1);
-  if (b >= total) return false;
-  uint64_t owner_mask = __ballot(b >= excl && b < incl);
-  int owner = __ffsll((unsigned long long)owner_mask) - 1;
+  s.nb = mine;
+  s.incl = wave_incl_scan_dpp_i(mine);
+  s.total = __builtin_amdgcn_readlane(s.incl, WAVE - 1);
+  return s;
+}
+__device__ __forceinline__ bool row_blocks_find(const RowBlockScan& s, const int32_t* __restrict__ offsets, int G,
+                                                int extra_rows, int BM, int b, RowBlock& rb) {
+  if (b < 0 || b >= s.total) return false;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int excl = s.incl - s.nb;
+  const uint64_t owner_mask = __ballot(b >= excl && b < s.incl);
+  const int owner = __ffsll((unsigned long long)owner_mask) - 1;
+  if (s.small) {
+    const int o_start = __builtin_amdgcn_readlane(s.start, owner);
+    const int o_c = __builtin_amdgcn_readlane(s.c, owner);
+    const int o_excl = __builtin_amdgcn_readlane(excl, owner);
+    rb.group = owner;
+    rb.row0 = o_start + (b - o_excl) * BM;
+    rb.nrows = min(BM, o_c - (b - o_excl) * BM);
+    return true;
+  }
+  const int Gt = G + (extra_rows > 0 ? 1 : 0);
+  const int per = (Gt + WAVE - 1) / WAVE;
+  const int g0 = lane * per;
   int grp = -1, row0 = 0, nrows = 0;
   if (lane == owner) {
     int acc = excl;
@@ -270,4 +287,9 @@ __device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offse
   rb.row0 = __builtin_amdgcn_readlane(row0, owner);
   rb.nrows = __builtin_amdgcn_readlane(nrows, owner);
   return true;
+}
+__device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offsets, int G, int extra_rows, int BM,
+                                               int b, RowBlock& rb) {
+  const RowBlockScan s = row_blocks_scan(offsets, G, extra_rows, BM);
+  return row_blocks_find(s, offsets, G, extra_rows, BM, b, rb);
 }

@@ -50,6 +50,10 @@ struct GemmArgs {
   int out_dtype;
   int32_t* acc_dbg;    // [M_cap, N], nullable
   int tile_gx, tile_gy, tile_pc;  // tile kernel: column tiles, row blocks (worst case), columns of a patch
+  int tile_slots;                 // tile kernel: blocks the chip runs at once
+  int tile_split_max;             // tile kernel: most shares a tile of the last partial round is split into
+  int32_t* tail_cnt;              // tile kernel: arrival counters of the split tiles (zero at launch), or null
+  int32_t* tail_part;             // tile kernel: partial accumulators of the split tiles
   int32_t* part;       // GEMM1 stream kernel: [S, M_cap, N] partial accumulators (split-k)
   int S;               // number of k splits (grid.z)
   int64_t M_cap;
@@ -611,25 +615,71 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   c.wm = c.w / WN;
   c.wn = c.w % WN;
   const int lane = c.lane, w = c.w, wm = c.wm, wn = c.wn;
-  // Workgroups go to the 8 XCDs (each with its own L2) round-robin by their linear id, and about one
-  // block per CU is resident at a time.  Tile coordinates are therefore dealt so that the blocks an
-  // XCD runs together form compact patches of TILE_PR row blocks x tile_pc column tiles: the tiles
-  // of a patch share their row panels and (inside an expert) their weight panels in that L2.
+  // ---- which tile, and which share of its reduction
+  // Real tiles (row blocks that exist x column tiles) get the ids [0, n_real) in three runs:
+  //   A: whole patches of TILE_PR row blocks x tile_pc column tiles, in rounds of 8 dealt to the 8 XCDs
+  //      (workgroups go to the XCDs, each with its own L2, round-robin by their linear id, so the
+  //      tiles an XCD runs together share their row panels and, inside an expert, their weight
+  //      panels in that L2);
+  //   B: the whole patches that do not fill a round of 8, one after the other;
+  //   C: the row blocks past the last whole patch row, row by row.
+  // With n_real tiles on `tile_slots` block slots the last n_real % tile_slots tiles would run alone
+  // on a nearly idle chip.  When they are at most half a round, each of them is split S ways along the
+  // reduction: the tile's own block takes the first share, helper blocks with ids past n_real the
+  // others.  Every share stores its int32 partial accumulators; whoever arrives last at the tile's
+  // counter adds the others' to its own (integer sums: the order cannot matter) and runs the
+  // epilogue.  Nobody waits for anybody.
   constexpr int TILE_PR = 4;
-  int bx, by;
+  const RowBlockScan scan = row_blocks_scan(a.offsets, a.G, a.extra_rows, BM);
+  const int nk_all = a.Kdim / 64;
+  int bx, by, split = 1, share = 0, tail_tile = -1;
   {
-    const unsigned id = blockIdx.x, xcd = id & 7u, j = id >> 3;
-    const unsigned per_patch = TILE_PR * a.tile_pc;
-    const unsigned patch = (j / per_patch) * 8u + xcd, q = j % per_patch;
-    const unsigned npc = a.tile_gx / a.tile_pc;  // patches across the columns
-    by = (int)((patch / npc) * TILE_PR + q / a.tile_pc);
-    bx = (int)((patch % npc) * a.tile_pc + q % a.tile_pc);
-    if (by >= a.tile_gy) return;
+    const int gx = a.tile_gx, pc = a.tile_pc, npc = gx / pc, per_patch = TILE_PR * pc;
+    const int RB = scan.total;
+    const int n_real = RB * gx;
+    const int bulk_rows = RB / TILE_PR * TILE_PR;
+    const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
+    const int nA = patches8 * per_patch, nB = (patches - patches8) * per_patch;
+    int left = 0;
+    if (a.tail_part != nullptr && a.tile_slots > 0) {
+      left = n_real % a.tile_slots;
+      if (left > 0 && 2 * left <= a.tile_slots) split = min(min(a.tile_split_max, a.tile_slots / left), nk_all);
+      if (split < 2) { split = 1; left = 0; }
+    }
+    int id = (int)blockIdx.x;
+    if (id >= n_real) {
+      const int h = id - n_real;
+      if (split == 1 || h >= left * (split - 1)) return;
+      tail_tile = h / (split - 1);
+      share = 1 + h % (split - 1);
+      id = n_real - left + tail_tile;
+    } else if (split > 1 && id >= n_real - left) {
+      tail_tile = id - (n_real - left);
+    }
+    if (id < nA + nB) {
+      int patch, q;
+      if (id < nA) {
+        const int xcd = id & 7, j = id >> 3;
+        patch = (j / per_patch) * 8 + xcd;
+        q = j % per_patch;
+      } else {
+        patch = patches8 + (id - nA) / per_patch;
+        q = (id - nA) % per_patch;
+      }
+      by = (patch / npc) * TILE_PR + q / pc;
+      bx = (patch % npc) * pc + q % pc;
+    } else {
+      by = bulk_rows + (id - nA - nB) / gx;
+      bx = (id - nA - nB) % gx;
+    }
   }
   RowBlock rb;
-  if (!find_row_block(a.offsets, a.G, a.extra_rows, BM, by, rb)) return;
+  if (!row_blocks_find(scan, a.offsets, a.G, a.extra_rows, BM, by, rb)) return;
+  // this block's k-steps [k_first, k_first + nk64)
+  const int k_first = (tail_tile >= 0) ? share * nk_all / split : 0;
+  const int k_end = (tail_tile >= 0) ? (share + 1) * nk_all / split : nk_all;
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
-  const int nk64 = a.Kdim / 64;
+  const int nk64 = k_end - k_first;
   const int I = (KIND == 1) ? a.N / 2 : 0;
   const int8_t* wbase = (g < a.G) ? a.w + (size_t)g * a.Kdim * a.N : a.w_extra;
   const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
@@ -644,10 +694,11 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   for (int i = 0; i < AP; ++i) {
     int rr = (AP * w + i) * 16 + (lane & 15);
     if (rr >= nrows) rr = 0;  // rows past the end alias the first row; their results are not stored
-    c.asrc[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (lane >> 4) * 16;
+    c.asrc[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k_first * 64 + (lane >> 4) * 16;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) c.bsrc[i] = wbase + (size_t)strip_of(2 * w + i) * nk64 * 1024 + lane * 16;
+  for (int i = 0; i < 2; ++i)
+    c.bsrc[i] = wbase + ((size_t)strip_of(2 * w + i) * nk_all + k_first) * 1024 + lane * 16;
   // the first two k-steps are requested as soon as their addresses exist; everything else the block
   // has to set up overlaps with their flight
   const int last = nk64 - 1;
@@ -686,6 +737,45 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // ---- epilogue (the stage buffers are free now: the bf16 rows of GEMM2 are staged there, two
   // wavefronts per buffer)
   __syncthreads();  // every wavefront is done reading the last stage; the row scales written at the start are visible
+  if (tail_tile >= 0) {
+    // one share of a split tile: publish the partial sums, count in, and only the last one goes on
+    __shared__ int s_last;
+    constexpr int WAVE_INTS = 8 * 16 * WAVE;           // accumulator words of one wavefront
+    constexpr int TILE_INTS = 2 * WN * WAVE_INTS;
+    // The partial sums go out and come in as device-scope accesses (they pass the XCD's L2 instead of
+    // living in it), so no cache has to be written back or invalidated as a whole around the counter.
+    int32_t* mine = a.tail_part + ((size_t)tail_tile * split + share) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+      if (mt < c.mt_count) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            __hip_atomic_store(mine + ((mt * 2 + t) * 16 + i) * WAVE, acc[mt][t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    // every store of this wavefront is acknowledged before the block counts in
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) s_last = (atomicAdd(a.tail_cnt + tail_tile, 1) == split - 1);
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    for (int s2 = 0; s2 < split; ++s2) {
+      if (s2 == share) continue;
+      const int32_t* theirs = a.tail_part + ((size_t)tail_tile * split + s2) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+        if (mt < c.mt_count) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+              acc[mt][t][i] += __hip_atomic_load(theirs + ((mt * 2 + t) * 16 + i) * WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+  }
   uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
   tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wm, wn, bx, row0, nrows, wsc, I);
 #endif
@@ -866,8 +956,32 @@ int tile_wn(int kind, int units) {
   return (want == 4 && units % wide == 0) ? 4 : 2;
 }
 
+// Scratch of the split tiles of a launch: arrival counters, then one slot of partial accumulators per
+// share.  At most `tile_slots` shares exist (splits x split tiles <= slots), a slot is the 256 x 64*WN
+// int32 tile of a block, and the slot count is capped so that the area has one size for every shape.
+constexpr size_t TILE_TAIL_CNT_BYTES = 4096;
+constexpr size_t TILE_TAIL_PART_BYTES = (size_t)64 << 20;
+constexpr size_t TILE_TAIL_BYTES = TILE_TAIL_CNT_BYTES + TILE_TAIL_PART_BYTES;
+
+__global__ void zero_words_kernel(int32_t* p, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0;
+}
+
+// compute units of the current device (asked once per device)
+int device_cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    cached[dev] = n > 0 ? n : -1;
+  }
+  return cached[dev] > 0 ? cached[dev] : 0;
+}
+
 template <int KIND>
-void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
+void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, size_t tail_bytes, hipStream_t st) {
   const int BM = 256;
   GemmArgs a = a0;
   const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
@@ -877,9 +991,26 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
   a.tile_pc = 1;
   for (int c = 1; c <= 8; ++c)
     if (a.tile_gx % c == 0) a.tile_pc = c;
-  // whole patches (4 row blocks x tile_pc column tiles), dealt to the XCDs in rounds of 8
-  const int64_t patches = (int64_t)((a.tile_gy + 3) / 4) * (a.tile_gx / a.tile_pc);
-  const int64_t nblocks = (patches + 7) / 8 * 8 * 4 * a.tile_pc;
+  // one block per real tile (the kernel numbers them from the row counts in device memory; ids past
+  // the real tiles leave at once) plus, when the last partial round is split, up to one round of helpers
+  int64_t nblocks = (int64_t)a.tile_gy * a.tile_gx;
+  a.tile_slots = 0;
+  a.tail_cnt = nullptr;
+  a.tail_part = nullptr;
+  const int cus = device_cu_count();
+  if (tail_ws && tail_bytes >= TILE_TAIL_BYTES && cus > 0 && env_int("OMNI_MOE_TILE_TAIL", 1)) {
+    const size_t slot_bytes = (size_t)2 * wn * 8 * 16 * WAVE * sizeof(int32_t);
+    const int blocks_per_cu = (wn == 4) ? 1 : 2;
+    int slots = cus * blocks_per_cu;
+    if ((size_t)slots * slot_bytes > TILE_TAIL_PART_BYTES) slots = (int)(TILE_TAIL_PART_BYTES / slot_bytes);
+    if ((size_t)slots * sizeof(int32_t) > TILE_TAIL_CNT_BYTES) slots = (int)(TILE_TAIL_CNT_BYTES / sizeof(int32_t));
+    a.tile_slots = slots;
+    a.tile_split_max = env_int("OMNI_MOE_TILE_SPLIT", 4);
+    a.tail_cnt = (int32_t*)tail_ws;
+    a.tail_part = (int32_t*)((char*)tail_ws + TILE_TAIL_CNT_BYTES);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, st, a.tail_cnt, slots);
+    nblocks += slots;
+  }
   dim3 grid((unsigned)nblocks), block(128 * wn);
   const bool bfi = KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE);
   if (wn == 4) {
@@ -892,10 +1023,11 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
 }
 
 template <int KIND>
-int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, hipStream_t st, const char* what) {
+int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, void* tail_ws, size_t tail_bytes, hipStream_t st,
+                  const char* what) {
   const int units = (KIND == 1) ? a.N / 32 : a.N / 16;
   if (p.tile) {
-    launch_tile<KIND>(a, M_cap, units, st);
+    launch_tile<KIND>(a, M_cap, units, tail_ws, tail_bytes, st);
   } else {
     const int mt = p.mt, nt = p.nt, d = p.d;
     if (units % (4 * nt) != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: %d output strips not divisible by %d", what, units, 4 * nt);
@@ -919,7 +1051,8 @@ int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, hipStream_t s
 
 size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
   if (p.tile) {
-    return (size_t)M_cap * I * sizeof(float) + 256;  // y = silu(gate) * up before the row quantiser
+    // y = silu(gate) * up before the row quantiser, then the scratch of the split tiles
+    return align256((size_t)M_cap * I * sizeof(float) + 256) + TILE_TAIL_BYTES;
   }
   return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
 }
@@ -968,7 +1101,8 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
     // fused epilogue: y = silu(gate)*up to scratch, then the row quantiser
     float* y = (float*)workspace;
     a.y = y;
-    rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
+    void* tail_ws = (char*)workspace + align256((size_t)M_cap * I * sizeof(float) + 256);
+    rc = dispatch_gemm<1>(a, p, M_cap, tail_ws, TILE_TAIL_BYTES, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
     dim3 qgrid((unsigned)((M_cap + 3) / 4)), qblock(256);
@@ -982,7 +1116,7 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   // split-k stream kernel: raw int32 partial sums, then one row kernel does the whole epilogue
   if (I > 256 * 16) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gemm1: intermediate size %d > 4096 in the small-batch path", I);
   a.part = (int32_t*)workspace;
-  rc = dispatch_gemm<1>(a, p, M_cap, st, "gemm1");
+  rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, st, "gemm1");
   if (rc) return rc;
   if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
   // few rows (decode): more threads per row shorten the per-thread chain of exp / divide sequences
@@ -998,7 +1132,8 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
 extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed,
                                       const float* w2_scale, const int8_t* w2_extra, const float* w2_extra_scale,
                                       int extra_rows, const int32_t* offsets, int G, int H, int I, int64_t M_cap,
-                                      int out_dtype, void* rows_out, int32_t* acc_dbg, void* stream) {
+                                      int out_dtype, void* rows_out, int32_t* acc_dbg, void* workspace, size_t ws_bytes,
+                                      void* stream) {
   int rc = check_group_args("gemm2", offsets, G, H, I, M_cap, extra_rows, w2_extra, w2_extra_scale);
   if (rc) return rc;
   if (M_cap == 0) return OMNI_OK;
@@ -1013,7 +1148,14 @@ extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, c
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = I; a.N = H; a.flags = 0;
   a.rows_out = rows_out; a.out_dtype = out_dtype; a.acc_dbg = acc_dbg; a.S = 1; a.M_cap = M_cap;
   Plan p = make_plan<2>(a.T, a.K, G, extra_rows, I, H, M_cap);
-  return dispatch_gemm<2>(a, p, M_cap, (hipStream_t)stream, "gemm2");
+  if (workspace && ((uintptr_t)workspace % 256)) OMNI_FAIL(OMNI_E_INVALID, "gemm2: workspace must be 256-byte aligned");
+  return dispatch_gemm<2>(a, p, M_cap, workspace, workspace ? ws_bytes : 0, (hipStream_t)stream, "gemm2");
+}
+
+extern "C" size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int H, int I) {
+  if (M_cap < 0 || I <= 0 || H <= 0 || G < 0) return 0;
+  Plan p = make_plan<2>((int)M_cap, 1, G, extra_rows, I, H, M_cap);
+  return p.tile ? TILE_TAIL_BYTES : 0;
 }
 
 extern "C" int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N, int8_t* packed,

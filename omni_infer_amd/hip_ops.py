@@ -265,7 +265,8 @@ def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_
 def grouped_gemm2_dequant(h_q: torch.Tensor, h_scale: torch.Tensor, w2_packed: torch.Tensor, w2_scale: torch.Tensor,
                           offsets: torch.Tensor, H: int, I: int, out_dtype: torch.dtype = torch.bfloat16,
                           extra: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, extra_rows: int = 0,
-                          want_acc: bool = False, out: Optional[torch.Tensor] = None):
+                          want_acc: bool = False, out: Optional[torch.Tensor] = None,
+                          workspace: Optional[torch.Tensor] = None):
     """GEMM2 + dequant: ``npu_grouped_matmul(scale=, per_token_scale=, output_dtype=bf16)``
     (fused_moe.py:570-574, :681-685).  Returns (rows [M_cap, H], acc)."""
     _need_gpu(h_q, h_scale, w2_packed, w2_scale, offsets)
@@ -275,9 +276,13 @@ def grouped_gemm2_dequant(h_q: torch.Tensor, h_scale: torch.Tensor, w2_packed: t
     rows = out if out is not None else torch.zeros(M_cap, H, dtype=out_dtype, device=dev)
     acc = torch.zeros(M_cap, H, dtype=torch.int32, device=dev) if want_acc else None
     ew, es = extra if extra is not None else (None, None)
+    need = L.lib().omni_moe_gemm2_workspace_bytes(G, extra_rows, M_cap, H, I)
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     rc = L.lib().omni_moe_gemm2_dequant(_ptr(h_q), _ptr(h_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(ew), _ptr(es),
                                         extra_rows, _ptr(offsets), G, H, I, M_cap, _DT[out_dtype], _ptr(rows),
-                                        _ptr(acc), _stream())
+                                        _ptr(acc), _ptr(workspace), workspace.numel() if workspace is not None else 0,
+                                        _stream())
     L.check(rc, "omni_moe_gemm2_dequant")
     return rows, acc
 

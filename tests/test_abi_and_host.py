@@ -67,7 +67,7 @@ def test_argument_validation_returns_codes(lib):
                                            None, p, 1 << 30, None) == -2                                # I % 64
     assert lib.omni_moe_gemm1_swiglu_quant(p, p, None, 0, 4, 1, p, p, None, None, 0, p, 1, 7168, 2048, 4, 0, p, p,
                                            None, p, 16, None) == -3
-    assert lib.omni_moe_gemm2_dequant(p, p, p, p, None, None, 0, p, 1, 7168, 2048, 4, 5, p, None, None) == -1
+    assert lib.omni_moe_gemm2_dequant(p, p, p, p, None, None, 0, p, 1, 7168, 2048, 4, 5, p, None, None, 0, None) == -1
     assert lib.omni_moe_combine(p, 1, p, p, 0, 0, 4, 100, 64, None, None, None, p, None) == -2          # K > 64
     assert lib.omni_moe_w8a8_layer(p, -1, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, p,
                                    p, 1 << 30, None) == -1                                              # int8 w/o scale
@@ -78,9 +78,12 @@ def test_workspace_sizes(lib):
     assert lib.omni_moe_permute_workspace_bytes(8192, 8, 32) == (64 + 1) * 257 * 4
     m_cap = 64 * 8 + 64
     assert lib.omni_moe_gemm1_workspace_bytes(64, 8, 32, 64, m_cap, 7168, 2048) >= m_cap * 2048 * 4 + m_cap * 4
-    # prefill-sized: the fp32 y = silu(gate) * up matrix, not the int32 gate/up planes
+    # prefill-sized: the fp32 y = silu(gate) * up matrix (not the int32 gate/up planes) plus the 64 MiB
+    # scratch of the tiles whose reduction is shared between blocks
     big = lib.omni_moe_gemm1_workspace_bytes(8192, 8, 32, 8192, 73728, 7168, 2048)
-    assert 73728 * 2048 * 4 <= big < 73728 * 2048 * 4 + (1 << 20)
+    assert 73728 * 2048 * 4 + (64 << 20) <= big < 73728 * 2048 * 4 + (65 << 20)
+    assert lib.omni_moe_gemm2_workspace_bytes(32, 8192, 73728, 7168, 2048) == (64 << 20) + 4096
+    assert lib.omni_moe_gemm2_workspace_bytes(32, 64, 576, 7168, 2048) == 0
     total = lib.omni_moe_w8a8_layer_workspace_bytes(64, 8, 32, 7168, 2048, 1)
     assert total >= m_cap * (2048 + 2048 * 4 + 7168 * 4)
     assert total % 256 == 0

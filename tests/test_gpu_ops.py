@@ -186,6 +186,8 @@ def _grouped_case(T, K, n_local, E, H, I, seed, lo=0):
     (300, 4, 4, 8, 1024, 512, 1),       # ragged groups > 64 rows through the stream kernel
     (300, 4, 4, 8, 1024, 512, 2),       # same through the tile kernel
     (1100, 4, 3, 6, 512, 256, 0),       # tile kernel by default, partial 256-row blocks
+    (700, 2, 3, 3, 1024, 512, 2),       # tile kernel, 24 tiles per GEMM: each tile's reduction is shared by four blocks
+    (520, 1, 1, 1, 2048, 1024, 2),      # one group of three row blocks: 24 / 96 tiles, split four ways / two ways
 ])
 def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, monkeypatch):
     from omni_infer_amd import _lib as L
@@ -212,6 +214,33 @@ def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, monkeypatch):
     rows32, _ = ops.grouped_gemm2_dequant(h_q, h_s, d["w2"], d["s2"], p.offsets, H, I, out_dtype=torch.float32)
     out = ops.moe_combine(rows32, w.cuda(), p.src_to_dst, L.OMNI_IDX_TOKEN_MAJOR, L.OMNI_ORDER_SLOT)
     _eq(out, out_ref, "combined output")
+
+
+def test_split_tiles_equal_unsplit(ops, monkeypatch):
+    """Tiles of the last partial round share their reduction between blocks (integer partial sums, the
+    last block to arrive adds them): the results are the same bits as with the sharing switched off."""
+    from omni_infer_amd import _lib as L
+    T, K, n_local, E, H, I = 700, 2, 3, 3, 1024, 512
+    lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 77)
+    d = lay.to_device()
+    p = ops.moe_permute(ids.cuda(), 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    monkeypatch.setenv("OMNI_MOE_FORCE_KERNEL", "2")
+    got = {}
+    for tail in ("1", "0"):
+        monkeypatch.setenv("OMNI_MOE_TILE_TAIL", tail)
+        for rep in range(3):   # repeated launches reuse the same scratch and counters
+            h_q, h_s, acc1 = ops.grouped_gemm1_swiglu_quant(xq.cuda(), xs.cuda(), p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K,
+                                                            d["w13"], d["s13"], p.offsets, H, I, T * K, want_acc=True)
+            rows, acc2 = ops.grouped_gemm2_dequant(h_q, h_s, d["w2"], d["s2"], p.offsets, H, I,
+                                                   out_dtype=torch.bfloat16, want_acc=True)
+            cur = [t.cpu() for t in (h_q, h_s, acc1, rows, acc2)]
+            if tail in got:
+                for a, b in zip(cur, got[tail]):
+                    assert torch.equal(a, b), "launches of the same call differ"
+            got[tail] = cur
+    for a, b, what in zip(got["1"], got["0"], ("h_q", "h_s", "acc1", "rows", "acc2")):
+        m = int(p.offsets[-1])
+        assert torch.equal(a[:m], b[:m]), f"{what}: split and unsplit tiles differ"
 
 
 def test_combine_k_order_with_skip(ops):
