@@ -41,6 +41,8 @@ OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_PROLOGUE, OMNI_GEMM1_NO_REQUANT = 1,
 OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 
+ABI_VERSION = 2   # omni_moe_abi_version() of the header these signatures were written from
+
 _lib = None
 
 
@@ -64,6 +66,10 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)  # AttributeError if the library does not export it
             fn.restype = res
             fn.argtypes = args
+        have = handle.omni_moe_abi_version()
+        if have != ABI_VERSION:
+            raise OmniMoeError(f"{LIB_PATH} has ABI version {have}, this package binds version {ABI_VERSION}: "
+                               "rebuild it with `python -m omni_infer_amd._build`")
         _lib = handle
     return _lib
 
