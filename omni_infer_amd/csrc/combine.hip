@@ -34,33 +34,39 @@ struct CombineArgs {
   uint16_t* out;
 };
 
+// VEC columns of one row as floats: 16 bytes per lane (4 fp32 or 8 bf16), element by element at a ragged end.
 // STREAM: the row is read once and not again (expert rows), so it need not stay in the caches
-template <int DT, bool STREAM = false>
-__device__ __forceinline__ void load4(const void* base, size_t row, int H, int c, int ncol, float* v) {
+template <int DT, bool STREAM, int VEC>
+__device__ __forceinline__ void load_vec(const void* base, size_t row, int H, int c, int ncol, bool vec, float* v) {
   if constexpr (DT == OMNI_DT_F32) {
+    static_assert(VEC == 4, "16 bytes of fp32");
     const float* p = (const float*)base + row * H + c;
-    if (ncol == 4) {
+    if (ncol == VEC && vec) {
       v4f t = STREAM ? __builtin_nontemporal_load((const v4f*)p) : *(const v4f*)p;
-      v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = t[j];
     } else {
-      for (int j = 0; j < 4; ++j) v[j] = j < ncol ? p[j] : 0.0f;
+      for (int j = 0; j < VEC; ++j) v[j] = j < ncol ? p[j] : 0.0f;
     }
   } else {
+    static_assert(VEC == 8, "16 bytes of bf16");
     const uint16_t* p = (const uint16_t*)base + row * H + c;
-    if (ncol == 4) {
-      v2i t = STREAM ? __builtin_nontemporal_load((const v2i*)p) : *(const v2i*)p;
-      v[0] = bf16_to_f32((uint16_t)((uint32_t)t[0] & 0xffffu));
-      v[1] = bf16_to_f32((uint16_t)((uint32_t)t[0] >> 16));
-      v[2] = bf16_to_f32((uint16_t)((uint32_t)t[1] & 0xffffu));
-      v[3] = bf16_to_f32((uint16_t)((uint32_t)t[1] >> 16));
+    if (ncol == VEC && vec) {
+      v4i t = STREAM ? __builtin_nontemporal_load((const v4i*)p) : *(const v4i*)p;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = bf16_to_f32((uint16_t)((uint32_t)t[j] & 0xffffu));
+        v[2 * j + 1] = bf16_to_f32((uint16_t)((uint32_t)t[j] >> 16));
+      }
     } else {
-      for (int j = 0; j < 4; ++j) v[j] = j < ncol ? bf16_to_f32(p[j]) : 0.0f;
+      for (int j = 0; j < VEC; ++j) v[j] = j < ncol ? bf16_to_f32(p[j]) : 0.0f;
     }
   }
 }
 
 template <int DT>
 __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
+  constexpr int VEC = (DT == OMNI_DT_F32) ? 4 : 8;   // columns per thread and step
   __shared__ int s_slot[KMAX], s_raw[KMAX];
   __shared__ float s_w[KMAX];
   const int n = blockIdx.x;
@@ -91,46 +97,60 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
     }
   }
   __syncthreads();
+  const size_t post_row = (size_t)n + ((a.post_add && a.post_add_row0) ? (size_t)*a.post_add_row0 : 0);
+  const bool vec = (a.H % VEC) == 0;  // every row then starts on a 16-byte boundary
   // a block walks the column chunks blockIdx.y, blockIdx.y + gridDim.y, ... of its token
-  for (int c = (blockIdx.y * 256 + threadIdx.x) * 4; c < a.H; c += gridDim.y * 1024) {
-  const int ncol = min(4, a.H - c);
-  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (a.init) load4<OMNI_DT_BF16>(a.init, (size_t)n, a.H, c, ncol, acc);
-  // eight rows are requested together, then added in list order (one multiply, one add per row)
-  for (int j0 = 0; j0 < cnt; j0 += 8) {
-    float v[8][4];
+  for (int c = (blockIdx.y * 256 + threadIdx.x) * VEC; c < a.H; c += gridDim.y * 256 * VEC) {
+    const int ncol = min(VEC, a.H - c);
+    float acc[VEC];
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
-      if (j0 + u < cnt) load4<DT, true>(a.rows, (size_t)s_slot[j0 + u], a.H, c, ncol, v[u]);
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+    if (a.init) {
+      const uint16_t* ip = a.init + (size_t)n * a.H + c;
+      for (int j = 0; j < ncol; ++j) acc[j] = bf16_to_f32(ip[j]);
+    }
+    // the row added after the rounding is requested with the first batch
+    float pv[VEC];
+    if (a.post_add) load_vec<DT, false, VEC>(a.post_add, post_row, a.H, c, ncol, vec, pv);
+    // eight rows are requested together, then added in list order (one multiply, one add per row)
+    for (int j0 = 0; j0 < cnt; j0 += 8) {
+      float v[8][VEC];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      if (j0 + u < cnt) {
-        const float wv = s_w[j0 + u];
+      for (int u = 0; u < 8; ++u)
+        if (j0 + u < cnt) load_vec<DT, true, VEC>(a.rows, (size_t)s_slot[j0 + u], a.H, c, ncol, vec, v[u]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float prod = wv * v[u][i];
-          acc[i] = acc[i] + prod;
+      for (int u = 0; u < 8; ++u) {
+        if (j0 + u < cnt) {
+          const float wu = s_w[j0 + u];
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) {
+            float prod = wu * v[u][i];
+            acc[i] = acc[i] + prod;
+          }
         }
       }
     }
-  }
-  uint16_t o[4];
+    uint16_t o[VEC];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(acc[i]);
-  if (a.post_add) {
-    float v[4];
-    size_t r = (size_t)n + (a.post_add_row0 ? (size_t)*a.post_add_row0 : 0);
-    load4<DT>(a.post_add, r, a.H, c, ncol, v);
+    for (int i = 0; i < VEC; ++i) o[i] = f32_to_bf16(acc[i]);
+    if (a.post_add) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16(bf16_to_f32(o[i]) + round_bf16(v[i]));
-  }
-  uint16_t* op = a.out + (size_t)n * a.H + c;
-  if (ncol == 4) {
-    v2i t = {(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
-    *(v2i*)op = t;
-  } else {
-    for (int j = 0; j < ncol; ++j) op[j] = o[j];
-  }
+      for (int i = 0; i < VEC; ++i) o[i] = f32_to_bf16(bf16_to_f32(o[i]) + round_bf16(pv[i]));
+    }
+    uint16_t* op = a.out + (size_t)n * a.H + c;
+    if (ncol == VEC && vec) {
+      if constexpr (VEC == 4) {
+        v2i t = {(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
+        *(v2i*)op = t;
+      } else {
+        v4i t;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] = (int)((uint32_t)o[2 * j] | ((uint32_t)o[2 * j + 1] << 16));
+        *(v4i*)op = t;
+      }
+    } else {
+      for (int j = 0; j < ncol; ++j) op[j] = o[j];
+    }
   }
 }
 
@@ -146,13 +166,16 @@ extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* t
   if (!rows || !topk_w || !src_to_dst || !out_bf16) OMNI_FAIL(OMNI_E_INVALID, "combine: null pointer");
   if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "combine: rows_dtype %d", rows_dtype);
   if (H % 4 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "combine: H=%d must be a multiple of 4", H);
-  if (((uintptr_t)rows % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)init_bf16 % 8) || ((uintptr_t)post_add % 16))
+  // a thread moves 16 bytes of a row at a time: 4 fp32 or 8 bf16 columns in, as many bf16 columns out
+  const uintptr_t out_align = (rows_dtype == OMNI_DT_BF16) ? 16 : 8;
+  if (((uintptr_t)rows % 16) || ((uintptr_t)out_bf16 % out_align) || ((uintptr_t)post_add % 16))
     OMNI_FAIL(OMNI_E_INVALID, "combine: misaligned pointer");
   CombineArgs a{rows, rows_dtype, topk_w, src_to_dst, idx_mode, order, T, K, H, (const uint16_t*)init_bf16, post_add,
                 post_add_row0, (uint16_t*)out_bf16};
-  // few tokens: one block per (token, 1024-column chunk) for parallelism; many tokens: one block per
-  // token walks all chunks, so that a row's bytes are requested close together in time
-  const unsigned chunks = (unsigned)((H + 1023) / 1024);
+  // few tokens: one block per (token, chunk of 256 x 16 bytes) for parallelism; many tokens: one block
+  // per token walks all chunks, so that a row's bytes are requested close together in time
+  const int chunk_cols = 256 * ((rows_dtype == OMNI_DT_BF16) ? 8 : 4);
+  const unsigned chunks = (unsigned)((H + chunk_cols - 1) / chunk_cols);
   dim3 grid((unsigned)T, T >= 2048 ? 1u : chunks), block(256);
   hipStream_t st = (hipStream_t)stream;
   if (rows_dtype == OMNI_DT_F32) hipLaunchKernelGGL(combine_kernel<OMNI_DT_F32>, grid, block, 0, st, a);
