@@ -305,11 +305,14 @@ def test_full_size_properties(env, T):
 
 
 # ------------------------------------------------------------------ HIP graph capture of the call sequence
-def test_layer_call_sequence_is_graph_capturable(env):
+@pytest.mark.parametrize("T", [64, 600])
+def test_layer_call_sequence_is_graph_capturable(env, T):
     """Router + whole-layer entry captured in a HIP graph (no allocation, synchronisation or host read
     inside the library), replayed three times with eager work and synchronisations in between; every
-    replay must give the bits of the eager run, also after the inputs changed in place."""
-    T, K, E, n, H, I = 64, 8, 32, 4, 1024, 512
+    replay must give the bits of the eager run, also after the inputs changed in place.  64 tokens run
+    the stream kernels; 600 tokens the tile kernel, whose few tiles share their reductions between
+    blocks through counters that every launch clears with a kernel of its own."""
+    K, E, n, H, I = 8, 32, 4, 1024, 512
     lay = Layer(n, H, I, seed=77, shared=True)
     d = lay.to_device()
     g = gen(78)
