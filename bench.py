@@ -34,7 +34,7 @@ INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/cl
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (scaled by what the same counters read for the 1 GiB copies of --copy-probe); the summaries with
 # the full commands are profiles/decode_gemm1_hbm_traffic.txt and profiles/prefill_gemm1_hbm_traffic.txt.
-MEASURED_TRAFFIC = {"decode": 994_443_000, "prefill": 6_447_616_000}
+MEASURED_TRAFFIC = {"decode": 987_888_000, "prefill": 6_447_616_000}
 
 SHAPES = {
     "decode": dict(T=64, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5, outlier=0.0),
@@ -304,8 +304,8 @@ def main():
     k_ms = e0.elapsed_time(e1) / ksteps
     rows_total = rows_routed + T
     if args.workload == "decode":
-        # weights of every active group + the int8 tokens + the int32 accumulators the kernel writes
-        k_alg = active * (H * 2 * I) + T * H + rows_total * 2 * I * 4
+        # weights of every active group + the int8 tokens + the fp32 y = silu(gate)*up the kernel writes
+        k_alg = active * (H * 2 * I) + T * H + rows_total * I * 4
         roof = dict(bound="hbm", kernel="gemm_stream<1,2,1,4>", achieved=k_alg / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9,
                     unit="GB/s")
     else:

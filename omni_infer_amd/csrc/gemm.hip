@@ -221,6 +221,38 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
   // ---- epilogue
   const int col = lane & 15;
   if constexpr (KIND == 1) {
+    if (a.y != nullptr) {
+      // a single k share: the wavefront holds the gate and the up sums of its channels, so it
+      // dequantises and applies SwiGLU here; the row quantiser is left with the maximum and the rounding
+      const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt < mt_cnt) {
+          const int rbase = mt * 16 + 4 * (lane >> 4);
+          float ts[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            ts[i] = (rbase + i < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rbase + i)] : 0.0f;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const int n = strip[2 * t] * 16 + col;
+            const float wg = wsc[n], wu = wsc[I + n];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (rbase + i < nrows) {
+                float dg = ((float)acc[mt][2 * t][i] * wg) * ts[i];
+                float du = ((float)acc[mt][2 * t + 1][i] * wu) * ts[i];
+                if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+                float yv = silu_spec(dg) * du;
+                if (bf) yv = round_bf16(yv);
+                a.y[(size_t)(row0 + rbase + i) * I + n] = yv;
+              }
+            }
+          }
+        }
+      }
+      return;
+    }
     // raw int32 partial sums of this k share; the row kernel adds the shares and finishes
     int32_t* part = a.part + (size_t)blockIdx.z * a.M_cap * a.N;
 #pragma unroll
@@ -1057,6 +1089,15 @@ size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
   return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
 }
 
+void launch_quant_rows_y(const float* y, const int32_t* offsets, int G, int extra_rows, int I, int64_t M_cap,
+                         int8_t* h_q, float* h_scale, hipStream_t st) {
+  dim3 qgrid((unsigned)((M_cap + 3) / 4)), qblock(256);
+  if (I <= 256 * 4) hipLaunchKernelGGL(quant_rows_y<4>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+  else if (I <= 256 * 8) hipLaunchKernelGGL(quant_rows_y<8>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+  else if (I <= 256 * 16) hipLaunchKernelGGL(quant_rows_y<16>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+  else hipLaunchKernelGGL(quant_rows_y<0>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+}
+
 int check_group_args(const char* what, const int32_t* offsets, int G, int H, int I, int64_t M_cap, int extra_rows,
                      const void* w_extra, const void* w_extra_scale) {
   if (G < 0 || H <= 0 || I <= 0 || M_cap < 0 || extra_rows < 0) OMNI_FAIL(OMNI_E_INVALID, "%s: bad sizes G=%d H=%d I=%d M_cap=%lld", what, G, H, I, (long long)M_cap);
@@ -1105,11 +1146,18 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
     rc = dispatch_gemm<1>(a, p, M_cap, tail_ws, TILE_TAIL_BYTES, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
-    dim3 qgrid((unsigned)((M_cap + 3) / 4)), qblock(256);
-    if (I <= 256 * 4) hipLaunchKernelGGL(quant_rows_y<4>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
-    else if (I <= 256 * 8) hipLaunchKernelGGL(quant_rows_y<8>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
-    else if (I <= 256 * 16) hipLaunchKernelGGL(quant_rows_y<16>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
-    else hipLaunchKernelGGL(quant_rows_y<0>, qgrid, qblock, 0, st, y, offsets, G, extra_rows, I, M_cap, h_q, h_scale);
+    launch_quant_rows_y(y, offsets, G, extra_rows, I, M_cap, h_q, h_scale, st);
+    OMNI_CHECK_LAUNCH("gemm1 quant");
+    return OMNI_OK;
+  }
+  if (p.S == 1 && acc_dbg == nullptr) {
+    // one k share: the stream kernel finishes y = silu(gate)*up itself (the workspace holds it, half
+    // the bytes of the raw sums), then the row quantiser of the tile path
+    a.y = (float*)workspace;
+    rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, st, "gemm1");
+    if (rc) return rc;
+    if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
+    launch_quant_rows_y(a.y, offsets, G, extra_rows, I, M_cap, h_q, h_scale, st);
     OMNI_CHECK_LAUNCH("gemm1 quant");
     return OMNI_OK;
   }

@@ -205,6 +205,11 @@ def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, monkeypatch):
     _eq(acc1[:m], st["acc1"], "GEMM1 int32 accumulators")
     _eq(h_s[:m], st["h_s"], "stage-2 scales")
     _eq(h_q[:m], st["h_q"], "stage-2 int8 activations")
+    # without the accumulator dump the small-batch kernel applies SwiGLU itself: same bits
+    h_q2, h_s2, _ = ops.grouped_gemm1_swiglu_quant(xq.cuda(), xs.cuda(), p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K,
+                                                   d["w13"], d["s13"], p.offsets, H, I, M_cap)
+    _eq(h_s2[:m], st["h_s"], "stage-2 scales (no dump)")
+    _eq(h_q2[:m], st["h_q"], "stage-2 int8 activations (no dump)")
     for dt in (torch.float32, torch.bfloat16):
         rows, acc2 = ops.grouped_gemm2_dequant(h_q, h_s, d["w2"], d["s2"], p.offsets, H, I, out_dtype=dt, want_acc=True)
         _eq(acc2[:m], st["acc2"], "GEMM2 int32 accumulators")
