@@ -34,7 +34,7 @@ INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/cl
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (scaled by what the same counters read for the 1 GiB copies of --copy-probe); the summaries with
 # the full commands are profiles/decode_gemm1_hbm_traffic.txt and profiles/prefill_gemm1_hbm_traffic.txt.
-MEASURED_TRAFFIC = {"decode": 987_888_000, "prefill": 6_447_616_000}
+MEASURED_TRAFFIC = {"decode": 987_888_000, "prefill": 7_283_159_000}
 
 SHAPES = {
     "decode": dict(T=64, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5, outlier=0.0),
