@@ -226,7 +226,7 @@ def main():
     for s in sets[1:]:
         s.drop_ckpt()
     x, logits, bias = make_inputs(cfg, dev)
-    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, 1)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, 1, L.OMNI_DT_F32)
     workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
 
@@ -285,7 +285,7 @@ def main():
     g1_ws = torch.zeros(L.lib().omni_moe_gemm1_workspace_bytes(T, K, n_local, T, M_cap, H, I), dtype=torch.uint8, device=dev)
     hq = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
     hs = torch.empty(M_cap, dtype=torch.float32, device=dev)
-    kflags = L.OMNI_GEMM1_NO_PROLOGUE | L.OMNI_GEMM1_NO_REQUANT
+    kflags = L.OMNI_GEMM1_NO_REQUANT
 
     def gemm1_only(i):
         ws = sets[i % len(sets)]

@@ -56,7 +56,6 @@ extern "C" {
 /* gemm flags */
 #define OMNI_GEMM1_BF16_INTERMEDIATE 1 /* round the dequantised gate/up and the SwiGLU product to bf16
                                           (numerics of the non-EP pipeline, compressed_tensors_moe.py:242-247) */
-#define OMNI_GEMM1_NO_PROLOGUE 2  /* accepted and ignored: no kernel runs ahead of the GEMM any more */
 #define OMNI_GEMM1_NO_REQUANT 4   /* stop after the GEMM kernel: its result (int32 accumulators or fp32 y)
                                      stays in the workspace, h_q / h_scale are not written.  The call is then
                                      exactly one kernel launch, which is how the benchmark times that kernel
@@ -211,14 +210,20 @@ int omni_moe_combine(const void* rows, int rows_dtype, const float* topk_w, cons
  * (deepseek_moe.py:64-118,244,303) carried as an extra group.  Routing weights and ids are inputs
  * (omni_moe_route makes them).  x_dtype BF16: x is quantised first; x_dtype -1: x is int8 and
  * x_scale is given.  Returns bf16 [T,H].
+ *   rows_dtype is the caller's choice of how the expert rows travel from GEMM2 to the weighted sum:
+ *   OMNI_DT_F32  the rows stay fp32 and are rounded once, after the sum: the numerics of
+ *                npu_grouped_matmul_finalize_routing (fused_moe.py:536); 4*H bytes per row of workspace;
+ *   OMNI_DT_BF16 every row is rounded to bf16 first: the numerics of a bf16 npu_grouped_matmul followed by
+ *                npu_moe_finalize_routing (fused_moe.py:570-574 + deepseek_moe.py:292-301); half the bytes.
+ *   The same value must be given to omni_moe_w8a8_layer_workspace_bytes.
  */
 int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
                         const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
                         const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
                         const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
-                        const float* sh2_scale, int H, int I, void* out_bf16, void* workspace, size_t ws_bytes,
-                        void* stream);
-size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared);
+                        const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16, void* workspace,
+                        size_t ws_bytes, void* stream);
+size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared, int rows_dtype);
 
 #ifdef __cplusplus
 }

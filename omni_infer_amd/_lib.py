@@ -30,18 +30,18 @@ SIGNATURES = {
     "omni_moe_gemm2_dequant": (I, [P, P, P, P, P, P, I, P, I, I, I, c_int64, I, P, P, P, c_size_t, P]),
     "omni_moe_gemm2_workspace_bytes": (c_size_t, [I, I, c_int64, I, I]),
     "omni_moe_combine": (I, [P, I, P, P, I, I, I, I, I, P, P, P, P, P]),
-    "omni_moe_w8a8_layer": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, P, P, c_size_t, P]),
-    "omni_moe_w8a8_layer_workspace_bytes": (c_size_t, [I, I, I, I, I, I]),
+    "omni_moe_w8a8_layer": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
+    "omni_moe_w8a8_layer_workspace_bytes": (c_size_t, [I, I, I, I, I, I, I]),
 }
 
 OMNI_DT_BF16, OMNI_DT_F32, OMNI_DT_F16 = 0, 1, 2
 OMNI_SCORE_SOFTMAX, OMNI_SCORE_SIGMOID = 0, 1
 OMNI_GROUP_MAX, OMNI_GROUP_TOP2SUM = 0, 1
-OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_PROLOGUE, OMNI_GEMM1_NO_REQUANT = 1, 2, 4
+OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_REQUANT = 1, 4
 OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 
-ABI_VERSION = 2   # omni_moe_abi_version() of the header these signatures were written from
+ABI_VERSION = 3   # omni_moe_abi_version() of the header these signatures were written from
 
 _lib = None
 

@@ -16,7 +16,7 @@ void omni_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 extern "C" const char* omni_moe_last_error(void) { return g_err; }
-extern "C" int omni_moe_abi_version(void) { return 2; }
+extern "C" int omni_moe_abi_version(void) { return 3; }
 
 namespace {
 
@@ -192,12 +192,10 @@ struct LayerWs {
   int64_t M_cap;
   int rows_dtype;
 };
-// The expert rows between GEMM2 and the combine are kept in fp32 (the numerics of the fused
-// GEMM2+finalize operator) while that buffer stays within the 256 MiB last-level cache; beyond it
-// they are rounded to bf16 (the numerics of the separate GEMM2 and finalize operators), which
-// halves the largest intermediate of a prefill-sized call.
-constexpr size_t ROWS_F32_LIMIT = (size_t)256 << 20;
-LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
+// rows_dtype: the caller's choice for the expert rows between GEMM2 and the combine, fp32 (the
+// numerics of the fused GEMM2+finalize operator) or bf16 (those of the separate GEMM2 and finalize
+// operators, half the bytes of the largest intermediate).
+LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared, int rows_dtype) {
   LayerWs L{};
   L.M_cap = (int64_t)T * K + (with_shared ? T : 0);
   size_t o = 0;
@@ -216,25 +214,28 @@ LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared) {
   const size_t g2_bytes = omni_moe_gemm2_workspace_bytes(G, with_shared ? T : 0, L.M_cap, H, I);
   if (g2_bytes > L.g1_bytes) L.g1_bytes = g2_bytes;
   L.g1_ws = take(L.g1_bytes);
-  L.rows_dtype = ((size_t)L.M_cap * H * 4 <= ROWS_F32_LIMIT) ? OMNI_DT_F32 : OMNI_DT_BF16;
+  L.rows_dtype = rows_dtype;
   L.rows = take((size_t)L.M_cap * H * (L.rows_dtype == OMNI_DT_F32 ? 4 : 2));
   L.total = o;
   return L;
 }
 }  // namespace
 
-extern "C" size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared) {
+extern "C" size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared,
+                                                      int rows_dtype) {
   if (T < 0 || K <= 0 || n_local <= 0 || H <= 0 || I <= 0) return 0;
-  return layer_layout(T, K, n_local, H, I, with_shared).total;
+  if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) return 0;
+  return layer_layout(T, K, n_local, H, I, with_shared, rows_dtype).total;
 }
 
 extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
                                    const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
                                    const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
                                    const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
-                                   const float* sh2_scale, int H, int I, void* out_bf16, void* workspace,
-                                   size_t ws_bytes, void* stream) {
+                                   const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16,
+                                   void* workspace, size_t ws_bytes, void* stream) {
   if (T < 0 || K <= 0 || hi <= lo || H <= 0 || I <= 0) OMNI_FAIL(OMNI_E_INVALID, "layer: bad sizes");
+  if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "layer: rows_dtype %d", rows_dtype);
   if (T == 0) return OMNI_OK;
   if (!x || !topk_w || !topk_ids || !out_bf16 || !workspace) OMNI_FAIL(OMNI_E_INVALID, "layer: null pointer");
   if (x_dtype == -1 && !x_scale_in) OMNI_FAIL(OMNI_E_INVALID, "layer: int8 input without scales");
@@ -242,7 +243,7 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
   const int with_shared = sh13_packed != nullptr;
   if (with_shared && (!sh13_scale || !sh2_packed || !sh2_scale)) OMNI_FAIL(OMNI_E_INVALID, "layer: incomplete shared expert");
   if ((uintptr_t)workspace % 256) OMNI_FAIL(OMNI_E_INVALID, "layer: workspace must be 256-byte aligned");
-  LayerWs L = layer_layout(T, K, G, H, I, with_shared);
+  LayerWs L = layer_layout(T, K, G, H, I, with_shared, rows_dtype);
   if (ws_bytes < L.total) OMNI_FAIL(OMNI_E_WORKSPACE, "layer: workspace %zu < %zu", ws_bytes, L.total);
   char* ws = (char*)workspace;
   const int8_t* xq = (const int8_t*)x;

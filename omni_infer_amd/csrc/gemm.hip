@@ -1,30 +1,34 @@
-// Grouped int8 x int8 -> int32 GEMMs on v_mfma_i32_16x16x64_i8 with fused epilogues.
+// Grouped int8 x int8 -> int32 GEMMs on the gfx950 int8 MFMAs with fused epilogues.
 //
 // Operand layouts
 //   B (weights) is in the frag16 format: tiles of 16 output channels x 64 reduction elements,
-//   1 KiB each, in exactly the order the MFMA wants them in registers (lane l owns bytes
-//   [16 l, 16 l + 16) of a tile).  A 16-channel strip is contiguous along k, so a wavefront that
-//   walks k streams one contiguous region per strip with 16-byte loads.
+//   1 KiB each, in exactly the order v_mfma_i32_16x16x64_i8 wants them in registers (lane l owns
+//   bytes [16 l, 16 l + 16) of a tile).  A 16-channel strip is contiguous along k, so a wavefront
+//   that walks k streams one contiguous region per strip with 16-byte loads.  Two neighbouring
+//   strips hold the operands of v_mfma_i32_32x32x32_i8 as 256-byte runs.
 //   A (int8 activations) is row major in memory.  It is staged through LDS in the same fragment
 //   order: one wavefront load instruction fetches a 16 row x 64 byte fragment (lane l: row l%16,
 //   bytes 16*(l/16)..+16) and stores it linearly, so LDS writes and the later ds_read_b128
 //   fragment reads are both conflict free.  The gather by sorted slot (the permutation of the
 //   MoE) happens in this load: no sorted copy of the activations is ever made.
-//   C: lane l of a 16x16 tile holds rows 4*(l/16)..+4 of column l%16.
+//   C of a 16x16 tile: lane l holds rows 4*(l/16)..+4 of column l%16; of a 32x32 tile: column
+//   l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15.
 //
-// Two kernels share the epilogues:
-//   gemm_stream  rows per group <= 64 or so: weight streaming.  Each wavefront owns whole
-//                16-channel strips of B and loads them straight from global memory into MFMA
-//                registers through a ring of D outstanding k-steps (each weight byte is used by
-//                exactly one wavefront, so LDS staging would only add traffic); A is small and
-//                shared by the four wavefronts of a block through LDS.
-//   gemm_pipe    large row counts: 256 x 128 block tiles, A and B both loaded straight into LDS
-//                through a three-stage ring, each wavefront a 128 x 64 sub-tile on 32x32x32 MFMAs.
+// Two kernels share the epilogue arithmetic:
+//   gemm_stream  few rows per group (decode): weight streaming on the 16x16x64 MFMA.  Each
+//                wavefront owns whole 16-channel strips of B and loads them straight from global
+//                memory into MFMA registers through a ring of D outstanding k-steps (each weight
+//                byte is used by exactly one wavefront, so LDS staging would only add traffic); A
+//                is small and shared by the four wavefronts of a block through LDS.
+//   gemm_pipe    many rows per group (prefill): 256 x 256 (or 256 x 128) block tiles, A and B both
+//                loaded straight into LDS (global_load_lds) through a three-stage ring, each
+//                wavefront a 128 x 64 sub-tile on the 32x32x32 MFMA.
 //
 // GEMM1 pairs gate channel n with up channel I + n in the same lane so SwiGLU needs no exchange.
-// Its epilogue writes y = silu(gate) * up in fp32 to a scratch matrix and folds max|y| of each
-// row into a per-row word with an atomic max on the float's bit pattern (exact and order
-// independent for non-negative floats); a second small kernel quantises the rows.
+// Its epilogue writes y = silu(gate) * up in fp32 to a scratch matrix; a row kernel
+// (quant_rows_y) then takes max|y| of each row and quantises it.  With several k shares or when
+// the raw accumulators are asked for, gemm_stream stores int32 partial sums instead and
+// swiglu_quant_rows finishes them.
 #include "common.h"
 #include <type_traits>
 
@@ -774,8 +778,13 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     __shared__ int s_last;
     constexpr int WAVE_INTS = 8 * 16 * WAVE;           // accumulator words of one wavefront
     constexpr int TILE_INTS = 2 * WN * WAVE_INTS;
-    // The partial sums go out and come in as device-scope accesses (they pass the XCD's L2 instead of
-    // living in it), so no cache has to be written back or invalidated as a whole around the counter.
+    // Hand-over between the shares of a tile (their blocks may run on different XCDs, each with its own
+    // L2).  Every wavefront stores its partial sums, all wavefronts meet at the block barrier, then one
+    // thread counts in with a device-scope acquire-release add: the release half makes every store
+    // that happened before it (the barrier orders the other wavefronts' stores before it) visible to
+    // the device before the counter moves, and whoever reads the final count has, through the acquire
+    // half and the chain of adds on the same counter, all other shares' stores visible to its block
+    // after the second barrier.  No share ever waits for another.
     int32_t* mine = a.tail_part + ((size_t)tail_tile * split + share) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
@@ -783,17 +792,14 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int i = 0; i < 16; ++i)
-            __hip_atomic_store(mine + ((mt * 2 + t) * 16 + i) * WAVE, acc[mt][t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int i = 0; i < 16; ++i) mine[((mt * 2 + t) * 16 + i) * WAVE] = acc[mt][t][i];
       }
-    // every store of this wavefront is acknowledged before the block counts in
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
     __syncthreads();
-    if (threadIdx.x == 0) s_last = (atomicAdd(a.tail_cnt + tail_tile, 1) == split - 1);
+    if (threadIdx.x == 0)
+      s_last = (__hip_atomic_fetch_add(a.tail_cnt + tail_tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == split - 1);
     __syncthreads();
     if (!s_last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     for (int s2 = 0; s2 < split; ++s2) {
       if (s2 == share) continue;
       const int32_t* theirs = a.tail_part + ((size_t)tail_tile * split + s2) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
@@ -803,8 +809,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #pragma unroll
           for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
-              acc[mt][t][i] += __hip_atomic_load(theirs + ((mt * 2 + t) * 16 + i) * WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 0; i < 16; ++i) acc[mt][t][i] += theirs[((mt * 2 + t) * 16 + i) * WAVE];
         }
     }
   }
@@ -912,9 +917,60 @@ struct Plan {
   int64_t per;    // expected rows of a busy group
 };
 
-int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : dflt;
+// Tuning aids, read from the environment once (the first GEMM call of the process) and never again:
+//   OMNI_MOE_FORCE_KERNEL  1 stream kernel, 2 tile kernel, whatever the row counts
+//   OMNI_MOE_G1 / _G2      "mt,nt,d[,S]" of the stream kernel of GEMM1 / GEMM2; a combination that is not
+//                          compiled in is refused here, with a message, and the default is used
+//   OMNI_MOE_TILE_WN       2: tile kernel of 256 x 128 instead of 256 x 256
+//   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
+//   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
+//   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
+struct Tuning {
+  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0;
+  bool have[3] = {false, false, false};
+  int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
+};
+bool stream_variant_exists(int kind, int mt, int nt, int d);
+const Tuning& tuning() {
+  static const Tuning t = [] {
+    Tuning r;
+    auto geti = [](const char* name, int dflt) {
+      const char* v = getenv(name);
+      return v ? atoi(v) : dflt;
+    };
+    r.force_kernel = geti("OMNI_MOE_FORCE_KERNEL", 0);
+    r.tile_wn = geti("OMNI_MOE_TILE_WN", 4);
+    r.tile_tail = geti("OMNI_MOE_TILE_TAIL", 1);
+    r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
+    r.rowq = geti("OMNI_MOE_ROWQ", 0);
+    for (int kind = 1; kind <= 2; ++kind) {
+      const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
+      const char* e = getenv(name);
+      if (!e) continue;
+      int mt = 0, nt = 0, d = 0, S = 0;
+      if (sscanf(e, "%d,%d,%d,%d", &mt, &nt, &d, &S) >= 3 && stream_variant_exists(kind, mt, nt, d)) {
+        r.have[kind] = true;
+        r.mt[kind] = mt; r.nt[kind] = nt; r.d[kind] = d; r.S[kind] = S;
+      } else {
+        fprintf(stderr, "omni_moe: %s=\"%s\" names no compiled stream kernel; ignored\n", name, e);
+      }
+    }
+    return r;
+  }();
+  return t;
+}
+
+// the compiled (KIND, MT, NT, D) combinations of gemm_stream
+#define OMNI_STREAM_VARIANTS(X)                                                        \
+  X(1, 1, 1, 4) X(1, 2, 1, 4) X(1, 4, 1, 4) X(1, 1, 1, 8) X(1, 2, 1, 8)                \
+  X(1, 1, 2, 4) X(1, 2, 2, 4) X(1, 4, 2, 4) X(1, 2, 2, 8)                              \
+  X(2, 1, 1, 4) X(2, 2, 1, 4) X(2, 4, 1, 4) X(2, 1, 2, 4) X(2, 2, 2, 4) X(2, 4, 2, 4)  \
+  X(2, 1, 4, 4) X(2, 2, 4, 4) X(2, 2, 2, 8) X(2, 1, 2, 8) X(2, 2, 1, 8)
+bool stream_variant_exists(int kind, int mt, int nt, int d) {
+#define HAS(K_, MT_, NT_, D_) if (kind == K_ && mt == MT_ && nt == NT_ && d == D_) return true;
+  OMNI_STREAM_VARIANTS(HAS)
+#undef HAS
+  return false;
 }
 
 // Decides the kernel from what the host knows: the expected rows of a busy group.  The stream
@@ -934,7 +990,8 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
   // nearly every group is one block and its weights are read once; the shared group then takes a few
   // blocks and re-reads its 3 % of the bytes); above that the tile kernel does.
   p.tile = (G > 0) ? per > 48 : per > 128;
-  int force = env_int("OMNI_MOE_FORCE_KERNEL", 0);  // tuning aid: 1 stream, 2 tile
+  const Tuning& tn = tuning();
+  const int force = tn.force_kernel;
   if (force == 1) p.tile = false;
   if (force == 2) p.tile = true;
   const bool tile_ok = units % ((KIND == 1) ? 4 : 8) == 0;  // the tile kernel takes 64 / 128 channels at least
@@ -949,7 +1006,7 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
     p.nt = 1; p.d = 4;
   }
   int s_env = 0;
-  if (const char* e = getenv(KIND == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2")) sscanf(e, "%d,%d,%d,%d", &p.mt, &p.nt, &p.d, &s_env);
+  if (tn.have[KIND]) { p.mt = tn.mt[KIND]; p.nt = tn.nt[KIND]; p.d = tn.d[KIND]; s_env = tn.S[KIND]; }
   if (Kdim % (64 * p.d) != 0) p.d = 4;
   if (KIND == 1 && !p.tile && Kdim % 256 == 0 && units % (4 * p.nt) == 0) {
     const int nchunks = Kdim / 256, dc = p.d / 4;
@@ -957,7 +1014,7 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
     int64_t mb = (int64_t)Gt * ((per + 16 * p.mt - 1) / (16 * p.mt));
     int64_t base = (int64_t)(units / (4 * p.nt)) * (mb > 0 ? mb : 1);
     // measured on MI355X: extra k splits cost more in block start-up than they win back in the
-    // tail of the launch, so the default is one share; OMNI_MOE_G1="mt,nt,d,S" overrides
+    // tail of the launch, so the default is one share (the tuning aid OMNI_MOE_G1 can ask for more)
     int want = 1;
     (void)base;
     if (s_env > 0) want = s_env;
@@ -984,8 +1041,7 @@ void launch_stream(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) 
 // wavefront columns of the large tile: 4 (256 channels per block) when the channel count allows, else 2
 int tile_wn(int kind, int units) {
   const int wide = (kind == 1) ? 8 : 16;  // units per 256-channel block
-  const int want = env_int("OMNI_MOE_TILE_WN", 4);
-  return (want == 4 && units % wide == 0) ? 4 : 2;
+  return (tuning().tile_wn == 4 && units % wide == 0) ? 4 : 2;
 }
 
 // Scratch of the split tiles of a launch: arrival counters, then one slot of partial accumulators per
@@ -1030,14 +1086,14 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, si
   a.tail_cnt = nullptr;
   a.tail_part = nullptr;
   const int cus = device_cu_count();
-  if (tail_ws && tail_bytes >= TILE_TAIL_BYTES && cus > 0 && env_int("OMNI_MOE_TILE_TAIL", 1)) {
+  if (tail_ws && tail_bytes >= TILE_TAIL_BYTES && cus > 0 && tuning().tile_tail) {
     const size_t slot_bytes = (size_t)2 * wn * 8 * 16 * WAVE * sizeof(int32_t);
     const int blocks_per_cu = (wn == 4) ? 1 : 2;
     int slots = cus * blocks_per_cu;
     if ((size_t)slots * slot_bytes > TILE_TAIL_PART_BYTES) slots = (int)(TILE_TAIL_PART_BYTES / slot_bytes);
     if ((size_t)slots * sizeof(int32_t) > TILE_TAIL_CNT_BYTES) slots = (int)(TILE_TAIL_CNT_BYTES / sizeof(int32_t));
     a.tile_slots = slots;
-    a.tile_split_max = env_int("OMNI_MOE_TILE_SPLIT", 4);
+    a.tile_split_max = tuning().tile_split;
     a.tail_cnt = (int32_t*)tail_ws;
     a.tail_part = (int32_t*)((char*)tail_ws + TILE_TAIL_CNT_BYTES);
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, st, a.tail_cnt, slots);
@@ -1070,10 +1126,7 @@ int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, void* tail_ws
     if constexpr (KIND == K_) launch_stream<K_, MT_, NT_, D_>(a, M_cap, units, st); \
     ok = true;                                                                 \
   }
-    TRY(1, 1, 1, 4) TRY(1, 2, 1, 4) TRY(1, 4, 1, 4) TRY(1, 1, 1, 8) TRY(1, 2, 1, 8)
-    TRY(1, 1, 2, 4) TRY(1, 2, 2, 4) TRY(1, 4, 2, 4) TRY(1, 2, 2, 8)
-    TRY(2, 1, 1, 4) TRY(2, 2, 1, 4) TRY(2, 4, 1, 4) TRY(2, 1, 2, 4) TRY(2, 2, 2, 4) TRY(2, 4, 2, 4)
-    TRY(2, 1, 4, 4) TRY(2, 2, 4, 4) TRY(2, 2, 2, 8) TRY(2, 1, 2, 8) TRY(2, 2, 1, 8)
+    OMNI_STREAM_VARIANTS(TRY)
 #undef TRY
     if (!ok) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: no stream kernel variant mt=%d nt=%d d=%d", what, mt, nt, d);
   }
@@ -1168,7 +1221,7 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   if (rc) return rc;
   if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
   // few rows (decode): more threads per row shorten the per-thread chain of exp / divide sequences
-  const int rq = env_int("OMNI_MOE_ROWQ", M_cap <= 2048 ? 512 : 256);  // measured at 576 rows: 512 threads best
+  const int rq = tuning().rowq ? tuning().rowq : (M_cap <= 2048 ? 512 : 256);  // measured at 576 rows: 512 threads best
   if (I > 256 * 8) hipLaunchKernelGGL((swiglu_quant_rows<16, 256>), dim3((unsigned)M_cap), dim3(256), 0, st, a, h_q, h_scale);
   else if (rq == 1024 && I <= 1024 * 2) hipLaunchKernelGGL((swiglu_quant_rows<2, 1024>), dim3((unsigned)M_cap), dim3(1024), 0, st, a, h_q, h_scale);
   else if (rq >= 512 && I <= 512 * 4) hipLaunchKernelGGL((swiglu_quant_rows<4, 512>), dim3((unsigned)M_cap), dim3(512), 0, st, a, h_q, h_scale);

@@ -308,9 +308,16 @@ def moe_combine(rows: torch.Tensor, topk_w: torch.Tensor, src_to_dst: torch.Tens
 
 def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: torch.Tensor, topk_ids: torch.Tensor,
                    lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None, H: int = 0, I: int = 0,
-                   workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                   rows_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """The whole local-share layer in one library call (quant if x is bf16, permute, GEMM1
-    epilogue, GEMM2, combine), the shared expert carried as an extra group."""
+    epilogue, GEMM2, combine), the shared expert carried as an extra group.
+
+    ``rows_dtype`` is how the expert rows travel from GEMM2 to the weighted sum.  ``torch.float32``
+    (default) keeps them fp32 and rounds once after the sum: the numerics of
+    ``npu_grouped_matmul_finalize_routing`` (fused_moe.py:536).  ``torch.bfloat16`` rounds every row
+    first: the numerics of the bf16 ``npu_grouped_matmul`` + ``npu_moe_finalize_routing`` pair
+    (fused_moe.py:570-574, deepseek_moe.py:292-301), half the bytes of the largest intermediate."""
     _need_gpu(x, topk_w, topk_ids)
     T, K = topk_ids.shape
     dev = x.device
@@ -319,14 +326,16 @@ def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: tor
     topk_ids = topk_ids.to(torch.int32).contiguous()
     x_dtype = -1 if x.dtype == torch.int8 else _DT[x.dtype]
     sh = shared if shared is not None else (None, None, None, None)
-    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, hi - lo, H, I, int(shared is not None))
+    if rows_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("rows_dtype must be torch.float32 or torch.bfloat16")
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, hi - lo, H, I, int(shared is not None), _DT[rows_dtype])
     if workspace is None or workspace.numel() < need:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     if out is None:
         out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
     rc = L.lib().omni_moe_w8a8_layer(_ptr(x), x_dtype, _ptr(x_scale), _ptr(topk_w), _ptr(topk_ids), T, K, lo, hi,
                                      _ptr(w13_packed), _ptr(w13_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(sh[0]),
-                                     _ptr(sh[1]), _ptr(sh[2]), _ptr(sh[3]), H, I, _ptr(out), _ptr(workspace),
-                                     workspace.numel(), _stream())
+                                     _ptr(sh[1]), _ptr(sh[2]), _ptr(sh[3]), H, I, _DT[rows_dtype], _ptr(out),
+                                     _ptr(workspace), workspace.numel(), _stream())
     L.check(rc, "omni_moe_w8a8_layer")
     return out

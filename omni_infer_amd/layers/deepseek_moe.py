@@ -109,6 +109,10 @@ class DeepseekMoE(nn.Module):
                 prefix=f"{prefix}.shared_experts", device=device)
         self.local_expert_num = self.experts.w13_weight.shape[0]
         self.fused = True
+        # how the expert rows travel from GEMM2 to the weighted sum in the fused body: fp32 is what the
+        # reference's fused GEMM2+finalize operator accumulates from (fused_moe.py:536); torch.bfloat16
+        # halves the largest intermediate of a prefill-sized call at the price of one more rounding
+        self.rows_dtype = torch.float32
         self._workspace = None
 
     def process_weights_after_loading(self) -> None:
@@ -173,10 +177,12 @@ class DeepseekMoE(nn.Module):
             shared = (gu.weight, gu.weight_scale, dn.weight, dn.weight_scale)
         T, K = topk_ids.shape
         need = ops.L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, self.local_expert_num, e.hidden_size,
-                                                               e.intermediate_size_per_partition, int(shared is not None))
+                                                               e.intermediate_size_per_partition, int(shared is not None),
+                                                               ops._DT[self.rows_dtype])
         if self._workspace is None or self._workspace.numel() < need:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=hidden_states.device)
         x_in = hidden_states if x_int8 is None else x_int8
         return ops.moe_w8a8_layer(x_in, pertoken_scale, topk_weights, topk_ids, lo, lo + self.local_expert_num,
                                   e.w13_weight, e.w13_weight_scale, e.w2_weight, e.w2_weight_scale.float(), shared,
-                                  H=e.hidden_size, I=e.intermediate_size_per_partition, workspace=self._workspace)
+                                  H=e.hidden_size, I=e.intermediate_size_per_partition, workspace=self._workspace,
+                                  rows_dtype=self.rows_dtype)

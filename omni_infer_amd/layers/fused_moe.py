@@ -44,11 +44,13 @@ def fused_experts_w8a8_allgather_ep(hidden_states: torch.Tensor, pertoken_scale:
                                     w2: torch.Tensor, w1_scale: torch.Tensor, w2_scale: torch.Tensor,
                                     topk_weights: torch.Tensor, topk_ids: torch.Tensor, n_routed_experts: int,
                                     is_prefill: bool, max_num_deployed_expert_per_rank: int,
-                                    hidden_size: Optional[int] = None, intermediate_size: Optional[int] = None):
+                                    hidden_size: Optional[int] = None, intermediate_size: Optional[int] = None,
+                                    rows_dtype: torch.dtype = torch.float32):
     """fused_moe.py:489-538.  hidden_states is int8 [T,H] with pertoken_scale [T]; topk_ids
     are global expert ids; only this GPU's experts are computed.  Returns bf16 [T,H], or None
     when the expert-parallel share is the whole model (the reference has no else branch,
-    fused_moe.py:504)."""
+    fused_moe.py:504).  ``rows_dtype`` (not in the reference): fp32 expert rows into the weighted
+    sum, as the reference's fused GEMM2+finalize operator has them (:536), or bf16 rows."""
     redundancy = model_extra_config.parall_config.redundancy_shared_expert_num
     expert_parallel_size = get_ep_group().world_size - redundancy
     if expert_parallel_size <= 1:
@@ -58,7 +60,7 @@ def fused_experts_w8a8_allgather_ep(hidden_states: torch.Tensor, pertoken_scale:
     lo = (get_world_group().rank_in_group - redundancy) * max_num_deployed_expert_per_rank
     hi = lo + n_routed_experts
     return ops.moe_w8a8_layer(hidden_states, pertoken_scale, topk_weights, topk_ids, lo, hi, w1, w1_scale, w2,
-                              w2_scale.float(), None, H=H, I=I)
+                              w2_scale.float(), None, H=H, I=I, rows_dtype=rows_dtype)
 
 
 def moe_expert_quant_farword(sorted_tokens: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w1_scale: torch.Tensor,

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
         assert hasattr(lib, n), f"{n} declared in the header but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.omni_moe_abi_version() == _lib.ABI_VERSION == 2
+    assert lib.omni_moe_abi_version() == _lib.ABI_VERSION == 3
 
 
 def test_header_constants_match_binding():
@@ -69,8 +69,11 @@ def test_argument_validation_returns_codes(lib):
                                            None, p, 16, None) == -3
     assert lib.omni_moe_gemm2_dequant(p, p, p, p, None, None, 0, p, 1, 7168, 2048, 4, 5, p, None, None, 0, None) == -1
     assert lib.omni_moe_combine(p, 1, p, p, 0, 0, 4, 100, 64, None, None, None, p, None) == -2          # K > 64
-    assert lib.omni_moe_w8a8_layer(p, -1, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, p,
+    assert lib.omni_moe_w8a8_layer(p, -1, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, 1, p,
                                    p, 1 << 30, None) == -1                                              # int8 w/o scale
+    assert lib.omni_moe_w8a8_layer(p, 0, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, 2, p,
+                                   p, 1 << 30, None) == -1                                              # rows_dtype f16
+    assert lib.omni_moe_w8a8_layer_workspace_bytes(4, 8, 32, 7168, 2048, 1, 2) == 0
 
 
 def test_workspace_sizes(lib):
@@ -84,9 +87,15 @@ def test_workspace_sizes(lib):
     assert 73728 * 2048 * 4 + (64 << 20) <= big < 73728 * 2048 * 4 + (65 << 20)
     assert lib.omni_moe_gemm2_workspace_bytes(32, 8192, 73728, 7168, 2048) == (64 << 20) + 4096
     assert lib.omni_moe_gemm2_workspace_bytes(32, 64, 576, 7168, 2048) == 0
-    total = lib.omni_moe_w8a8_layer_workspace_bytes(64, 8, 32, 7168, 2048, 1)
+    from omni_infer_amd import _lib
+    total = lib.omni_moe_w8a8_layer_workspace_bytes(64, 8, 32, 7168, 2048, 1, _lib.OMNI_DT_F32)
     assert total >= m_cap * (2048 + 2048 * 4 + 7168 * 4)
     assert total % 256 == 0
+    # the row buffer is the caller's choice and nothing else: bf16 rows save exactly half of it, at any size
+    for T in (64, 8192):
+        f32 = lib.omni_moe_w8a8_layer_workspace_bytes(T, 8, 32, 7168, 2048, 1, _lib.OMNI_DT_F32)
+        b16 = lib.omni_moe_w8a8_layer_workspace_bytes(T, 8, 32, 7168, 2048, 1, _lib.OMNI_DT_BF16)
+        assert f32 - b16 == (T * 9) * 7168 * 2
 
 
 def test_python_errors_match_reference_types(lib):

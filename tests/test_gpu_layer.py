@@ -320,7 +320,7 @@ def test_layer_call_sequence_is_graph_capturable(env, T):
     logits = torch.randn(T, E, generator=g).cuda()
     bias = (torch.randn(E, generator=g) * 0.01).cuda()
     ops, L = env.ops, env.L
-    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n, H, I, 1)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n, H, I, 1, L.OMNI_DT_F32)
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     out = torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
     shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
