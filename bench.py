@@ -6,14 +6,18 @@ A step is one pass of the layer over one batch of synthetic tokens, inputs resid
     sort by expert  ->  int8 GEMM1 + dequant + SwiGLU + requant  ->  int8 GEMM2 + dequant  ->
     weighted combine + shared expert.
 Workloads (BASELINE.json configs):
-    decode   DeepSeek-V3 shape, 32 local experts of 256 + 1 shared expert, 64 tokens   (default)
+    decode   DeepSeek-V3 shape, 32 local experts of 256 + 1 shared expert, 64 tokens
     prefill  same layer, 8192 tokens with 0.1 % outlier channels x50
 Router logits are random over the 32 local experts and -30 elsewhere, so the router itself
 sends every token to 8 distinct local experts ("uniform random routing into local experts").
-The gate GEMM that makes the logits is not part of the step.
+The gate GEMM that makes the logits is not part of the step; `block_us` times the whole block
+(gate included) through DeepseekMoE.forward.
 
-Prints one JSON line: layer time, the roofline figure of the dominant kernel (GEMM1), and the
-CPU oracle timed on this box's host cores on a bounded sample.
+The default run measures both halves of the metric and prints one JSON line: the headline is the
+decode layer time with the roofline figure of its dominant kernel (GEMM1) and the CPU oracle timed on
+this box's host cores; the `prefill` object carries the 8192-token layer time, its share of the int8
+peak, the rooflines of both tile GEMM kernels and the deviation from the oracle.  `--workload decode`
+or `--workload prefill` runs one half only (profiling runs).
 """
 from __future__ import annotations
 
@@ -31,10 +35,13 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12       # B/s, MI355X published
 INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/clk x 2.4 GHz = 5.03e15)
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (scaled by what the same counters read for the 1 GiB copies of --copy-probe); the summaries with
-# the full commands are profiles/decode_gemm1_hbm_traffic.txt and profiles/prefill_gemm1_hbm_traffic.txt.
-MEASURED_TRAFFIC = {"decode": 987_888_000, "prefill": 7_283_159_000}
+# HBM-side bytes per launch of the GEMM1 kernels as recorded from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# of this file (scaled by what the same counters read for the 1 GiB copies of --copy-probe).  Counters cannot
+# be read from inside a timed run, so these are values of record, labelled with the summary they come from.
+RECORDED_TRAFFIC = {
+    ("decode", "gemm1"): (987_888_000, "profiles/decode_gemm1_hbm_traffic.txt"),
+    ("prefill", "gemm1"): (7_283_159_000, "profiles/prefill_gemm1_hbm_traffic.txt"),
+}
 
 SHAPES = {
     "decode": dict(T=64, H=7168, I=2048, E=256, n_local=32, K=8, n_group=8, topk_group=4, scale=2.5, outlier=0.0),
@@ -105,7 +112,7 @@ def algorithmic_ops_layer(cfg, rows_routed):
     return 2 * (rows_routed + T) * (H * 2 * I + I * H)
 
 
-def cpu_baseline(cfg, ws, x, logits, bias, sample_tokens):
+def cpu_baseline(cfg, ws, x, logits, bias, sample_tokens, rows_bf16=False):
     """The oracle's whole layer on the host cores, on the first `sample_tokens` tokens."""
     from oracle import moe_oracle as O
     torch.set_num_threads(os.cpu_count() or 1)
@@ -115,6 +122,12 @@ def cpu_baseline(cfg, ws, x, logits, bias, sample_tokens):
     xs, ls, b = x[:sample_tokens].cpu(), logits[:sample_tokens].cpu(), bias.cpu()
 
     def run():
+        if rows_bf16:   # the library's bf16-row option: the same block with every expert row rounded before the sum
+            w, ids = O.route_noaux_tc(ls, b, cfg["K"], cfg["n_group"], cfg["topk_group"], cfg["scale"])
+            xq, xsc = O.dynamic_quant(xs)
+            o = O.fused_experts_w8a8_allgather_ep(xq, xsc, routed[0], routed[2], routed[1], routed[3], w, ids,
+                                                  (0, cfg["n_local"]), rows_bf16=True)
+            return o + O.shared_expert_mlp(xs, *shared)
         return O.deepseek_moe_forward(xs, ls, b, routed, shared, cfg["K"], cfg["n_group"], cfg["topk_group"],
                                       cfg["scale"], (0, cfg["n_local"]))
     out = run()  # untimed first pass (thread pool, page faults)
@@ -189,14 +202,201 @@ def bench_norm(args):
     print(json.dumps(result))
 
 
+def time_steps(fn, steps, warmup):
+    """Average GPU time of `steps` calls of fn(i) after `warmup` untimed ones (events on torch's current
+    stream, which is the stream every library call is enqueued on), plus the host wall time per step."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return max(e0.elapsed_time(e1) / steps, 0.0), (time.perf_counter() - t0) * 1e3 / steps
+
+
+def single_step_spread(fn, n):
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for i, (a0, a1) in enumerate(evs):
+        a0.record()
+        fn(i)
+        a1.record()
+    torch.cuda.synchronize()
+    per = sorted(a0.elapsed_time(a1) * 1e3 for a0, a1 in evs)
+    return {"p10": per[int(0.1 * (n - 1))], "p50": per[(n - 1) // 2], "p90": per[int(0.9 * (n - 1))]}
+
+
+def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_steps=None):
+    """One workload: whole-layer time, both GEMM kernels alone, the byte / op counts of the routing that
+    the router produced, and (unless no_cpu) the oracle on a bounded sample of the same tokens."""
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+    cfg = SHAPES[name]
+    T, H, I, K, n_local = cfg["T"], cfg["H"], cfg["I"], cfg["K"], cfg["n_local"]
+    x, logits, bias = make_inputs(cfg, dev)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, 1, ops._DT[rows_dtype])
+    workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+
+    def step(i):
+        ws = sets[i % len(sets)]
+        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
+                                             cfg["scale"], 1e-20)
+        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
+                                  (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out,
+                                  rows_dtype=rows_dtype)
+
+    ms, wall_ms = time_steps(step, steps, warmup)
+    spread = single_step_spread(step, min(50, steps))
+
+    # routing actually produced (rows per local expert) for the byte / op counts
+    w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
+    p = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    counts = p.counts.cpu()
+    rows_routed = int(counts.sum())
+    active = int((counts > 0).sum()) + 1
+    rows_total = rows_routed + T
+    layer_bytes = algorithmic_bytes_layer(cfg, active)
+    layer_ops = algorithmic_ops_layer(cfg, rows_routed)
+
+    # ---- the two GEMM kernels alone, each timed with events on its stream.  GEMM1 is called with
+    # OMNI_GEMM1_NO_REQUANT, which stops after the GEMM kernel; the tile kernel is preceded by the one-block
+    # fill kernel that clears its split-tile counters (about 2 us, inside the figure)
+    M_cap = T * K + T
+    xq, xs = ops.npu_dynamic_quant(x)
+    g1_ws = torch.zeros(L.lib().omni_moe_gemm1_workspace_bytes(T, K, n_local, T, M_cap, H, I), dtype=torch.uint8, device=dev)
+    hq = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
+    hs = torch.empty(M_cap, dtype=torch.float32, device=dev)
+    rows = torch.empty(M_cap, H, dtype=rows_dtype, device=dev)
+
+    def gemm1_only(i):
+        ws = sets[i % len(sets)]
+        ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, ws.w13, ws.s13, p.offsets, H, I,
+                                       M_cap, extra=(ws.sh13, ws.sh_s13), extra_rows=T, flags=L.OMNI_GEMM1_NO_REQUANT,
+                                       workspace=g1_ws, out=(hq, hs))
+
+    def gemm2_only(i):
+        ws = sets[i % len(sets)]
+        ops.grouped_gemm2_dequant(hq, hs, ws.w2, ws.s2, p.offsets, H, I, out_dtype=rows_dtype,
+                                  extra=(ws.sh2, ws.sh_s2), extra_rows=T, out=rows, workspace=g1_ws)
+
+    ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, sets[0].w13, sets[0].s13, p.offsets,
+                                   H, I, M_cap, extra=(sets[0].sh13, sets[0].sh_s13), extra_rows=T, workspace=g1_ws,
+                                   out=(hq, hs))                       # real int8 rows for GEMM2 to read
+    ksteps = kernel_steps or max(10, steps // 2)
+    k1_ms, _ = time_steps(gemm1_only, ksteps, 5)
+    k2_ms, _ = time_steps(gemm2_only, ksteps, 5)
+    name1 = ops.gemm_kernel_name(1, T, K, n_local, T, M_cap, H, I)
+    name2 = ops.gemm_kernel_name(2, T, K, n_local, T, M_cap, H, I)
+    rows_bytes = 4 if rows_dtype == torch.float32 else 2
+    if name == "decode":
+        # weights and scales of every active group + the int8 tokens (intermediates are implementation traffic)
+        alg1 = active * (H * 2 * I + 2 * I * 4) + T * H
+        alg2 = active * (I * H + H * 4) + rows_total * I
+        roofs = [dict(bound="hbm", kernel=name1, achieved=alg1 / (k1_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
+                      kernel_us=k1_ms * 1e3, algorithmic_per_launch=alg1),
+                 dict(bound="hbm", kernel=name2, achieved=alg2 / (k2_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9, unit="GB/s",
+                      kernel_us=k2_ms * 1e3, algorithmic_per_launch=alg2)]
+    else:
+        alg1 = 2 * rows_total * H * 2 * I
+        alg2 = 2 * rows_total * I * H
+        roofs = [dict(bound="mfma", kernel=name1, achieved=alg1 / (k1_ms * 1e-3) / 1e12, peak=INT8_PEAK / 1e12,
+                      unit="TFLOP/s", kernel_us=k1_ms * 1e3, algorithmic_per_launch=alg1),
+                 dict(bound="mfma", kernel=name2, achieved=alg2 / (k2_ms * 1e-3) / 1e12, peak=INT8_PEAK / 1e12,
+                      unit="TFLOP/s", kernel_us=k2_ms * 1e3, algorithmic_per_launch=alg2)]
+    for r, key in zip(roofs, ("gemm1", "gemm2")):
+        r["frac"] = r["achieved"] / r["peak"]
+        rec = RECORDED_TRAFFIC.get((name, key))
+        r["traffic"] = rec[0] if rec else None
+        if rec:
+            r["traffic_source"] = rec[1]
+    res = {
+        "workload": f"DeepSeek-V3-shape W8A8 MoE layer, {name}: {T} tokens, {n_local} local experts of {cfg['E']} + 1 shared, "
+                    f"H={H}, I={I}, top-{K} grouped sigmoid routing",
+        "tokens": T, "rows_routed": rows_routed, "active_groups": active, "rows_dtype": str(rows_dtype).split(".")[-1],
+        "layer_us": ms * 1e3, "ms_per_step": ms, "steps": steps, "warmup": warmup,
+        "algorithmic_bytes": layer_bytes, "algorithmic_ops": layer_ops,
+        "hbm_frac": layer_bytes / (ms * 1e-3) / HBM_PEAK, "int8_frac": layer_ops / (ms * 1e-3) / INT8_PEAK,
+        "host_wall_ms_per_step": wall_ms, "single_step_us": spread,
+        "roofline_gemm1": roofs[0], "roofline_gemm2": roofs[1],
+    }
+    if not no_cpu:
+        sample = T if name == "decode" else 1024
+        dt, reps, ref = cpu_baseline(cfg, sets[0], x, logits, bias, sample, rows_dtype == torch.bfloat16)
+        got = step(0)[:sample].float().cpu()
+        torch.cuda.synchronize()
+        refd = ref.float()
+        res["cpu_baseline"] = {"value": dt * 1e6 * (T / sample), "unit": "us", "cores": torch.get_num_threads(),
+                               "kind": "port",
+                               "sample": f"oracle layer on the first {sample} of {T} tokens "
+                                         f"({reps} passes of {dt:.3f} s" + (", scaled by tokens)" if sample != T else ")"),
+                               "gpu_vs_oracle_rel_err": float((got - refd).norm() / refd.norm()),
+                               "gpu_vs_oracle_bit_exact": bool(torch.equal(got, refd))}
+    return res, step
+
+
+def measure_block(name, ws, steps, warmup, dev):
+    """The whole MoE block through DeepseekMoE.forward (gate GEMM, router, layer; fused body): what a model
+    pays per layer call.  Weights are those of one weight set (no rotation: about the cache-resident share
+    of 1.45 GB is served from the last-level cache, so this figure is a lower bound next to `value`)."""
+    import types
+    from omni_infer_amd import config, distributed
+    from omni_infer_amd.layers.deepseek_moe import DeepseekMoE
+    from omni_infer_amd.quantization.compressed_tensors import AscendCompressedTensorsConfig
+    cfg = SHAPES[name]
+    T, H, I, K, n_local, E = cfg["T"], cfg["H"], cfg["I"], cfg["K"], cfg["n_local"], cfg["E"]
+    config.update_model_extra_config(enable_moe_expert_parallel=True, moe_dispatch_combine=False,
+                                     prefill_dispatch_combine=False)
+    distributed.set_virtual_ep(E // n_local, 0)
+    mc = types.SimpleNamespace(hidden_size=H, n_routed_experts=E, num_experts_per_tok=K, moe_intermediate_size=I,
+                               n_shared_experts=1, n_group=cfg["n_group"], topk_group=cfg["topk_group"],
+                               norm_topk_prob=True, scoring_func="sigmoid", topk_method="noaux_tc",
+                               routed_scaling_factor=cfg["scale"], hidden_act="silu", first_k_dense_replace=3)
+    blk = DeepseekMoE(mc, AscendCompressedTensorsConfig(ignore=["gate"]), prefix="model.layers.3.mlp", device=dev)
+    g = torch.Generator(device=dev).manual_seed(7)
+    gate_w = torch.randn(E, H, generator=g, device=dev) * 0.02
+    gate_w[n_local:] = 0.0            # the other ranks' experts score sigmoid(0) + a negative bias: never chosen
+    blk.gate.weight.data.copy_(gate_w)
+    bias = torch.randn(E, generator=g, device=dev) * 0.01
+    bias[n_local:] -= 10.0
+    blk.gate.e_score_correction_bias.data.copy_(bias)
+    w13, w2, sw13, sw2 = ws.ckpt
+    ex, se = blk.experts, blk.shared_experts
+    ex.w13_weight.data.copy_(w13)
+    ex.w2_weight.data.copy_(w2)
+    ex.w13_weight_scale.data.copy_(ws.s13)
+    ex.w2_weight_scale.data.copy_(ws.s2)
+    se.gate_up_proj.weight.data.copy_(sw13)
+    se.gate_up_proj.weight_scale.data.copy_(ws.sh_s13.unsqueeze(-1))
+    se.down_proj.weight.data.copy_(sw2)
+    se.down_proj.weight_scale.data.copy_(ws.sh_s2.unsqueeze(-1))
+    blk.process_weights_after_loading()
+    x, _, _ = make_inputs(cfg, dev)
+
+    def step(i):
+        return blk(x, None, None, 3)
+    ms, wall_ms = time_steps(step, steps, warmup)
+    ids = blk._route(x)[1]
+    local = int(((ids >= 0) & (ids < n_local)).sum())
+    return {"block_us": ms * 1e3, "host_wall_ms_per_step": wall_ms, "steps": steps, "local_assignments": local,
+            "tokens": T}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=sorted(SHAPES) + ["norm"], default="decode",
-                    help="decode (default, the headline metric) / prefill: the MoE layer; norm: the RMSNorm+quant producer")
+    ap.add_argument("--steps", type=int, default=4000, help="timed decode steps (prefill runs steps/100, at least 10)")
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", choices=["all", "decode", "prefill", "norm"], default="all",
+                    help="all (default): decode headline + prefill object + block_us; decode / prefill: that half only; "
+                         "norm: the RMSNorm+quant producer")
+    ap.add_argument("--rows", choices=["f32", "bf16"], default="f32",
+                    help="row dtype between GEMM2 and the combine (the product default is f32)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-block", action="store_true", help="skip the DeepseekMoE.forward timing")
     ap.add_argument("--weight-sets", type=int, default=2, help="weight copies rotated between steps (cache defeat)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 1 GiB device copies first (a kernel of known traffic to scale HBM counters by)")
@@ -210,32 +410,17 @@ def main():
         sys.exit(2)
 
     if args.workload == "norm":
+        if args.steps == 4000:
+            args.steps, args.warmup = 200, 20
         return bench_norm(args)
 
-    from omni_infer_amd import _lib as L
-    from omni_infer_amd import hip_ops as ops
-
-    cfg = SHAPES[args.workload]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    T, H, I, K, n_local = cfg["T"], cfg["H"], cfg["I"], cfg["K"], cfg["n_local"]
-    if args.workload == "prefill" and args.steps == 200:
-        args.steps, args.warmup = 20, 3
-
+    rows_dtype = torch.float32 if args.rows == "f32" else torch.bfloat16
+    cfg = SHAPES["decode"]
     sets = [WeightSet(cfg, 100 + i, dev) for i in range(max(1, args.weight_sets))]
     for s in sets[1:]:
         s.drop_ckpt()
-    x, logits, bias = make_inputs(cfg, dev)
-    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, 1, L.OMNI_DT_F32)
-    workspace = torch.empty(need, dtype=torch.uint8, device=dev)
-    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
-
-    def step(i):
-        ws = sets[i % len(sets)]
-        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
-                                             cfg["scale"], 1e-20)
-        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
-                                  (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out)
 
     if args.copy_probe:
         src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
@@ -245,103 +430,43 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(args.steps):
-        step(i)
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms = e0.elapsed_time(e1) / args.steps
-    ms = max(ms, 0.0)
+    pre_steps = max(10, args.steps // 100)
+    dec = pre = None
+    if args.workload in ("all", "decode"):
+        dec, _ = measure_layer("decode", sets, args.steps, args.warmup, rows_dtype, args.no_cpu, dev)
+    if args.workload in ("all", "prefill"):
+        pre, _ = measure_layer("prefill", sets, pre_steps, 3, rows_dtype, args.no_cpu, dev, kernel_steps=pre_steps)
+        if args.workload == "all":
+            other = torch.bfloat16 if rows_dtype == torch.float32 else torch.float32
+            alt, _ = measure_layer("prefill", sets, pre_steps, 3, other, True, dev, kernel_steps=pre_steps)
+            pre["other_rows_dtype"] = {k: alt[k] for k in ("rows_dtype", "layer_us", "int8_frac")}
+            pre["other_rows_dtype"]["gemm2_kernel_us"] = alt["roofline_gemm2"]["kernel_us"]
 
-    # spread of single steps (each bracketed by its own event pair; not part of `value`)
-    nd = min(50, args.steps)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nd)]
-    for i, (a0, a1) in enumerate(evs):
-        a0.record()
-        step(i)
-        a1.record()
-    torch.cuda.synchronize()
-    per = sorted(a0.elapsed_time(a1) * 1e3 for a0, a1 in evs)
-    spread = {"p10": per[int(0.1 * (nd - 1))], "p50": per[(nd - 1) // 2], "p90": per[int(0.9 * (nd - 1))]}
-
-    # routing actually produced (rows per local expert) for the byte / op counts
-    w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
-    p = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
-    counts = p.counts.cpu()
-    rows_routed = int(counts.sum())
-    active = int((counts > 0).sum()) + 1
-    layer_bytes = algorithmic_bytes_layer(cfg, active)
-    layer_ops = algorithmic_ops_layer(cfg, rows_routed)
-
-    # ---- dominant kernel alone: GEMM1 (one launch per call), timed with events on its stream
-    M_cap = T * K + T
-    xq, xs = ops.npu_dynamic_quant(x)
-    g1_ws = torch.zeros(L.lib().omni_moe_gemm1_workspace_bytes(T, K, n_local, T, M_cap, H, I), dtype=torch.uint8, device=dev)
-    hq = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
-    hs = torch.empty(M_cap, dtype=torch.float32, device=dev)
-    kflags = L.OMNI_GEMM1_NO_REQUANT
-
-    def gemm1_only(i):
-        ws = sets[i % len(sets)]
-        ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, ws.w13, ws.s13, p.offsets, H, I,
-                                       M_cap, extra=(ws.sh13, ws.sh_s13), extra_rows=T, flags=kflags, workspace=g1_ws,
-                                       out=(hq, hs))
-    ksteps = max(10, args.steps // 2)
-    for i in range(5):
-        gemm1_only(i)
-    torch.cuda.synchronize()
-    e0.record()
-    for i in range(ksteps):
-        gemm1_only(i)
-    e1.record()
-    torch.cuda.synchronize()
-    k_ms = e0.elapsed_time(e1) / ksteps
-    rows_total = rows_routed + T
-    if args.workload == "decode":
-        # weights of every active group + the int8 tokens + the fp32 y = silu(gate)*up the kernel writes
-        k_alg = active * (H * 2 * I) + T * H + rows_total * I * 4
-        roof = dict(bound="hbm", kernel="gemm_stream<1,2,1,4>", achieved=k_alg / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK / 1e9,
-                    unit="GB/s")
-    else:
-        k_alg = 2 * rows_total * H * 2 * I
-        roof = dict(bound="mfma", kernel="gemm_pipe<1,4>", achieved=k_alg / (k_ms * 1e-3) / 1e12, peak=INT8_PEAK / 1e12,
-                    unit="TFLOP/s")
-    roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["kernel_us"] = k_ms * 1e3
-    roof["algorithmic_per_launch"] = k_alg
-    roof["traffic"] = MEASURED_TRAFFIC.get(args.workload)
-
+    head = dec if dec is not None else pre
     result = {
-        "metric": "moe_layer_latency", "value": ms * 1e3, "unit": "us", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"DeepSeek-V3-shape W8A8 MoE layer, {args.workload}: {T} tokens, {n_local} local experts "
-                               f"of {cfg['E']} + 1 shared, H={H}, I={I}, top-{K} grouped sigmoid routing",
-                   "tokens": T, "rows_routed": rows_routed, "active_groups": active, "weight_sets": len(sets)},
-        "layer": {"algorithmic_bytes": layer_bytes, "algorithmic_ops": layer_ops,
-                  "hbm_frac": layer_bytes / (ms * 1e-3) / HBM_PEAK, "int8_frac": layer_ops / (ms * 1e-3) / INT8_PEAK,
-                  "host_wall_ms_per_step": wall_ms, "single_step_us": spread},
-        "roofline": roof,
+        "metric": "moe_layer_latency", "value": head["layer_us"], "unit": "us", "n_gpus": 1, "steps": head["steps"],
+        "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": head["workload"], "tokens": head["tokens"], "rows_routed": head["rows_routed"],
+                   "active_groups": head["active_groups"], "weight_sets": len(sets), "rows_dtype": head["rows_dtype"]},
+        "layer": {k: head[k] for k in ("algorithmic_bytes", "algorithmic_ops", "hbm_frac", "int8_frac",
+                                       "host_wall_ms_per_step", "single_step_us")},
+        "roofline": head["roofline_gemm1"],
+        "roofline_gemm2": head["roofline_gemm2"],
     }
-    if not args.no_cpu:
-        sample = T if args.workload == "decode" else 1024
-        dt, reps, ref = cpu_baseline(cfg, sets[0], x, logits, bias, sample)
-        got = step(0)[:sample].float().cpu()
-        torch.cuda.synchronize()
-        refd = ref.float()
-        rel = float((got - refd).norm() / refd.norm())
-        result["cpu_baseline"] = {"value": dt * 1e6 * (T / sample), "unit": "us", "cores": torch.get_num_threads(),
-                                  "kind": "port",
-                                  "sample": f"oracle layer on the first {sample} of {T} tokens "
-                                            f"({reps} passes of {dt:.3f} s" + (", scaled by tokens)" if sample != T else ")"),
-                                  "gpu_vs_oracle_rel_err": rel,
-                                  "gpu_vs_oracle_bit_exact": bool(torch.equal(got, refd))}
+    if "cpu_baseline" in head:
+        result["cpu_baseline"] = head["cpu_baseline"]
+    if dec is not None and pre is not None:
+        result["prefill"] = {k: pre[k] for k in ("workload", "tokens", "rows_routed", "rows_dtype", "layer_us", "steps",
+                                                 "algorithmic_ops", "int8_frac", "single_step_us", "roofline_gemm1",
+                                                 "roofline_gemm2", "other_rows_dtype")}
+        if "cpu_baseline" in pre:
+            result["prefill"]["gpu_vs_oracle_rel_err"] = pre["cpu_baseline"]["gpu_vs_oracle_rel_err"]
+            result["prefill"]["gpu_vs_oracle_bit_exact"] = pre["cpu_baseline"]["gpu_vs_oracle_bit_exact"]
+            result["prefill"]["cpu_baseline"] = pre["cpu_baseline"]
+    if not args.no_block and args.workload == "all":
+        result["block_us"] = {"decode": measure_block("decode", sets[0], max(50, args.steps // 10), 10, dev),
+                              "prefill": measure_block("prefill", sets[0], pre_steps, 2, dev)}
     print(json.dumps(result))
 
 

@@ -192,6 +192,15 @@ int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, const int8_t
 size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int H, int I);
 
 /*
+ * Which GEMM kernel the two entry points above launch for a call of these sizes (kind 1: GEMM1 with the
+ * arguments of omni_moe_gemm1_swiglu_quant; kind 2: GEMM2, T and K unused), written to buf as the kernel's
+ * template name, e.g. "gemm_stream<1,2,1,4>" or "gemm_pipe<2,4>".  A diagnostic for benchmarks and profiles
+ * (no counterpart in the reference, whose kernels are chosen inside the closed operators).
+ */
+int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, char* buf,
+                              size_t buf_bytes);
+
+/*
  * Weighted un-permute.  Replaces the routing half of npu_grouped_matmul_finalize_routing
  * (fused_moe.py:536), npu_moe_finalize_routing (compressed_tensors_moe.py:253;
  * deepseek_moe.py:292-301) and the shared-expert add (deepseek_moe.py:303,366).

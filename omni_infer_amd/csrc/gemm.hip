@@ -1259,6 +1259,17 @@ extern "C" size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t 
   return p.tile ? TILE_TAIL_BYTES : 0;
 }
 
+extern "C" int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I,
+                                         char* buf, size_t buf_bytes) {
+  if ((kind != 1 && kind != 2) || !buf || buf_bytes == 0) OMNI_FAIL(OMNI_E_INVALID, "gemm_kernel_name: bad arguments");
+  if (M_cap < 0 || I <= 0 || H <= 0 || G < 0 || (kind == 1 && (T <= 0 || K <= 0))) OMNI_FAIL(OMNI_E_INVALID, "gemm_kernel_name: bad sizes");
+  const Plan p = (kind == 1) ? make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap)
+                             : make_plan<2>((int)M_cap, 1, G, extra_rows, I, H, M_cap);
+  if (p.tile) snprintf(buf, buf_bytes, "gemm_pipe<%d,%d>", kind, tile_wn(kind, kind == 1 ? 2 * I / 32 : H / 16));
+  else snprintf(buf, buf_bytes, "gemm_stream<%d,%d,%d,%d>", kind, p.mt, p.nt, p.d);
+  return OMNI_OK;
+}
+
 extern "C" int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N, int8_t* packed,
                                     void* stream) {
   if (G <= 0 || Kdim <= 0 || N <= 0) OMNI_FAIL(OMNI_E_INVALID, "pack_weight: bad sizes");

@@ -287,6 +287,15 @@ def grouped_gemm2_dequant(h_q: torch.Tensor, h_scale: torch.Tensor, w2_packed: t
     return rows, acc
 
 
+def gemm_kernel_name(kind: int, T: int, K: int, G: int, extra_rows: int, M_cap: int, H: int, I: int) -> str:
+    """Template name of the GEMM kernel the library launches for a call of these sizes (diagnostic)."""
+    import ctypes
+    buf = ctypes.create_string_buffer(64)
+    rc = L.lib().omni_moe_gemm_kernel_name(kind, T, K, G, extra_rows, M_cap, H, I, ctypes.addressof(buf), 64)
+    L.check(rc, "omni_moe_gemm_kernel_name")
+    return buf.value.decode()
+
+
 def moe_combine(rows: torch.Tensor, topk_w: torch.Tensor, src_to_dst: torch.Tensor, idx_mode: int, order: int,
                 init: Optional[torch.Tensor] = None, post_add: Optional[torch.Tensor] = None,
                 post_add_row0: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -339,3 +348,4 @@ def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: tor
                                      _ptr(workspace), workspace.numel(), _stream())
     L.check(rc, "omni_moe_w8a8_layer")
     return out
+

@@ -42,9 +42,19 @@ tests/test_oracle_pins.py):
 * moe_init_routing_v1/v2  permutation invariants, bincount, numpy stable
   argsort.
 * grouped_matmul_int32 .. fp64 matmul witness, per-expert loop.
-* dequant_swiglu_quant, grouped_matmul_dequant, finalize ... closed forms in
-  float64, and the end-to-end dense brute force (every token through every
-  selected expert without any permutation).
+* dequant_swiglu_quant, grouped_matmul_dequant, quant_matmul, swiglu_bf16,
+  finalize ... closed forms in float64 from the exact integer products (a
+  wrong group's scale, a missing per-token scale, swapped halves must fail),
+  and the end-to-end dense brute force (every token through every selected
+  expert without any permutation).
+* moe_expert_quant_forward ... permutation-free fp64 witness; its second
+  stage within one bf16 step of the fp64 closed form with the w2 scale it was
+  asked to use (a skipped bf16 rounding of that scale fails).
+* deepseek_moe_forward ... fp64 witness of the whole block built from the
+  transformers router, the dense brute force and an fp64 shared expert (a
+  wrong expert range or a missing shared expert fails); the rounding points
+  of the final add (bf16 + bf16) by composition with the block without a
+  shared expert.
 * add_rms_norm / add_rms_norm_dynamic_quant (the producer in front of the
   block) ... torch.nn.functional.rms_norm in float64 (library routine) within
   one bf16 step, closed forms on constant and zero rows, power-of-two scale
@@ -463,20 +473,27 @@ def grouped_matmul_dequant(a: torch.Tensor, w: torch.Tensor, w_scale: torch.Tens
 def grouped_matmul_finalize_routing(a: torch.Tensor, w: torch.Tensor, counts: torch.Tensor, w_scale: torch.Tensor,
                                     per_token_scale: torch.Tensor, shared_input: Optional[torch.Tensor],
                                     logit: torch.Tensor, row_index: torch.Tensor, output_bs: int,
-                                    shared_input_weight: float = 1.0, shared_input_offset: int = 0) -> torch.Tensor:
+                                    shared_input_weight: float = 1.0, shared_input_offset: int = 0,
+                                    rows_bf16: bool = False) -> torch.Tensor:
     """``npu_grouped_matmul_finalize_routing`` (fused_moe.py:536).
 
     out[row_index[m], :] += logit[m] * ((float(acc2[m,:]) * w_scale[g,:]) * s[m])
     accumulated in fp32 in ascending m, starting from
     shared_input_weight * float(shared_input) on rows
     [offset, offset + shared_input.shape[0]).  Returns fp32 [output_bs, H].
+
+    ``rows_bf16`` (the device library's bf16-row option, not a mode of the reference operator):
+    every dequantised row is rounded to bf16 before it is weighted, which is what a bf16
+    ``npu_grouped_matmul`` (fused_moe.py:570-574) hands to a finalize step.
     """
     acc = grouped_matmul_int32(a, w, counts)
     m = acc.shape[0]
     g = _group_of_rows(counts)[:m]
     v = acc.to(F32) * w_scale.to(F32)[g]
     v = v * per_token_scale.to(F32)[:m].unsqueeze(-1)
-    v = v * logit.to(F32)[:m].unsqueeze(-1)
+    if rows_bf16:
+        v = v.to(torch.bfloat16).to(F32)
+    v = logit.to(F32)[:m].unsqueeze(-1) * v
     out = torch.zeros(output_bs, w.shape[2], dtype=F32)
     if shared_input is not None:
         n = shared_input.shape[0]
@@ -560,7 +577,7 @@ def shared_expert_mlp(x: torch.Tensor, w_gate_up: torch.Tensor, s_gate_up: torch
 # Pipelines
 # --------------------------------------------------------------------------
 def fused_experts_w8a8_allgather_ep(x_int8, pertoken_scale, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids,
-                                    expert_range, shared_input=None, return_stages=False):
+                                    expert_range, shared_input=None, return_stages=False, rows_bf16=False):
     """``fused_experts_w8a8_allgather_ep`` (fused_moe.py:489-538): the local-share
     pipeline.  x_int8 [T,H]; w1 [E_loc,H,2I]; w2 [E_loc,I,H]; topk_ids are
     global ids; only ids in expert_range = [lo, hi) are computed here.
@@ -575,7 +592,7 @@ def fused_experts_w8a8_allgather_ep(x_int8, pertoken_scale, w1, w2, w1_scale, w2
     if shared_input is None:
         shared_input = torch.zeros(T, w2.shape[2], dtype=torch.bfloat16)
     out32 = grouped_matmul_finalize_routing(hq, w2, counts, w2_scale.float(), hs, shared_input, w_sorted,
-                                            row_index, T)
+                                            row_index, T, rows_bf16=rows_bf16)
     out = out32.to(torch.bfloat16)
     if return_stages:
         acc2 = grouped_matmul_int32(hq, w2, counts)

@@ -300,3 +300,180 @@ def test_golden_fixtures_reproduce():
     assert sorted(saved) == sorted(fresh)
     for k in saved:
         assert torch.equal(saved[k], fresh[k]), k
+
+
+# ------------------------------------------------------------------ direct pins of the dequantising GEMMs and bf16 SwiGLU
+def _bf16_steps(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in bf16 representable steps between two bf16 tensors."""
+    ai = a.contiguous().view(torch.int16).to(torch.int32)
+    bi = b.contiguous().view(torch.int16).to(torch.int32)
+    ai = torch.where(ai < 0, -(ai & 0x7fff), ai)
+    bi = torch.where(bi < 0, -(bi & 0x7fff), bi)
+    return (ai - bi).abs()
+
+
+def test_grouped_matmul_dequant_closed_form():
+    """o[m] = (acc[m] . w_scale[g(m)]) . s[m] in fp64 from the exact integer product: a wrong group's
+    scale, a missing per-token scale or a transposed weight must fail."""
+    g = gen(20)
+    K, N = 512, 96
+    a = torch.randint(-128, 128, (45, K), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (4, K, N), generator=g, dtype=torch.int8)
+    ws = torch.rand(4, N, generator=g) * 1e-3 + 1e-4
+    ts = torch.rand(45, generator=g) * 0.05 + 0.01
+    counts = torch.tensor([11, 0, 30, 4])
+    grp = torch.repeat_interleave(torch.arange(4), counts)
+    exact = torch.stack([a[m].double() @ w[grp[m]].double() for m in range(45)])
+    want = exact * ws.double()[grp] * ts.double().unsqueeze(1)
+    got32 = O.grouped_matmul_dequant(a, w, ws, ts, counts, torch.float32)
+    assert float(((got32.double() - want) / want.abs().clamp(min=1e-30)).abs().max()) < 3e-7   # two fp32 roundings
+    got16 = O.grouped_matmul_dequant(a, w, ws, ts, counts, torch.bfloat16)
+    assert int(_bf16_steps(got16, want.to(torch.bfloat16)).max()) <= 1
+    assert float((_bf16_steps(got16, want.to(torch.bfloat16)) == 0).float().mean()) > 0.99
+    # the mistakes this must catch
+    wrong_group = exact * ws.double()[(grp + 1) % 4] * ts.double().unsqueeze(1)
+    no_token_scale = exact * ws.double()[grp]
+    for bad in (wrong_group, no_token_scale):
+        assert rel_err(got32, bad) > 0.1
+    # rows of an empty group do not exist: 45 rows, group 1 contributes none
+    assert got32.shape == (45, N)
+
+
+def test_quant_matmul_closed_form():
+    g = gen(21)
+    x = torch.randint(-128, 128, (33, 256), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (256, 80), generator=g, dtype=torch.int8)
+    ws = torch.rand(80, generator=g) * 1e-3 + 1e-4
+    ts = torch.rand(33, generator=g) * 0.05 + 0.01
+    exact = x.double() @ w.double()
+    assert torch.equal(O.quant_matmul(x, w, ws, None, torch.int32).double(), exact)
+    got = O.quant_matmul(x, w, ws, ts, torch.bfloat16)
+    want = (exact * ws.double() * ts.double().unsqueeze(1)).to(torch.bfloat16)
+    assert int(_bf16_steps(got, want).max()) <= 1 and float((_bf16_steps(got, want) == 0).float().mean()) > 0.99
+    got_nots = O.quant_matmul(x, w, ws, None, torch.float32)
+    assert rel_err(got_nots, exact * ws.double()) < 1e-6
+    assert rel_err(got.float(), exact * ws.double()) > 0.1          # the per-token scale is applied
+    assert rel_err(got.float(), (x.double() @ w.double().flip(0)) * ws.double() * ts.double().unsqueeze(1)) > 0.1
+
+
+def test_swiglu_bf16_closed_form():
+    g = gen(22)
+    x = (torch.randn(64, 512, generator=g) * 3).to(torch.bfloat16)
+    got = O.swiglu_bf16(x)
+    xd = x.double()
+    want = (xd[:, :256] / (1 + torch.exp(-xd[:, :256])) * xd[:, 256:])
+    steps = _bf16_steps(got, want.to(torch.bfloat16))
+    assert int(steps.max()) <= 1 and float((steps == 0).float().mean()) > 0.99   # one rounding at the end
+    swapped = (xd[:, 256:] / (1 + torch.exp(-xd[:, 256:])) * xd[:, :256])
+    assert rel_err(got.float(), swapped) > 0.1                                   # gate is the first half
+    assert got.dtype == torch.bfloat16 and got.shape == (64, 256)
+
+
+# ------------------------------------------------------------------ pipelines: grouped-rows form and the whole block
+def _fp64_expert_rows(rows_q, row_scale, w1, s1, w2, s2, counts):
+    """Permutation-free fp64 witness of the grouped-rows pipeline: one expert at a time, exact integer
+    products, SwiGLU and both quantisation steps in float64.  Returns (rows fp64 [M,H], y fp64)."""
+    M = rows_q.shape[0]
+    out = torch.zeros(M, w2.shape[2], dtype=torch.float64)
+    ys = torch.zeros(M, w1.shape[2] // 2, dtype=torch.float64)
+    start = 0
+    for e, c in enumerate(counts.tolist()):
+        if c == 0:
+            continue
+        sl = slice(start, start + c)
+        d = (rows_q[sl].double() @ w1[e].double()) * s1[e].double() * row_scale[sl].double().unsqueeze(1)
+        inter = d.shape[1] // 2
+        y = d[:, :inter] / (1 + torch.exp(-d[:, :inter])) * d[:, inter:]
+        s = y.abs().amax(1) / 127.0
+        q = torch.round(y / torch.where(s > 0, s, torch.ones_like(s)).unsqueeze(1)).clamp(-128, 127)
+        out[sl] = (q @ w2[e].double()) * s2[e].double() * s.unsqueeze(1)
+        ys[sl] = y
+        start += c
+    return out, ys
+
+
+@pytest.mark.parametrize("bf16_scale", [False, True])
+def test_moe_expert_quant_forward_against_fp64_witness(bf16_scale):
+    """moe_expert_quant_farword / gmm_expert (fused_moe.py:541-575, 663-687): rows grouped by expert.
+    (a) whole pipeline against the fp64 witness (int8 rounding flips bound the agreement);
+    (b) the second stage alone, fed the oracle's own int8 rows, must land within one bf16 step of the
+    fp64 closed form *with the w2 scale it was asked to use*: a skipped (or unasked-for) bf16 rounding of
+    the scale moves the rows by ~2^-9 and fails;  (c) wrong group boundaries fail."""
+    lay = Layer(5, 512, 256, seed=30)
+    g = gen(31)
+    counts = torch.tensor([9, 0, 23, 1, 14])
+    M = int(counts.sum())
+    x = tokens(M, 512, 31)
+    rows_q, rows_s = O.dynamic_quant(x)
+    got = O.moe_expert_quant_forward(rows_q, lay.w1_t, lay.w2_t, lay.s13, lay.s2, counts, rows_s, w2_scale_bf16=bf16_scale)
+    assert got.dtype == torch.bfloat16 and got.shape == (M, 512)
+    s2_used = lay.s2.to(torch.bfloat16).float() if bf16_scale else lay.s2
+    s2_other = lay.s2 if bf16_scale else lay.s2.to(torch.bfloat16).float()
+    wit, _ = _fp64_expert_rows(rows_q, rows_s, lay.w1_t, lay.s13, lay.w2_t, s2_used, counts)
+    assert rel_err(got.float(), wit) < 6e-3 and cosine(got.float(), wit) > 0.9999
+    # (b) stage 2 from the oracle's stage-1 output (both stage functions have pins of their own)
+    acc1 = O.grouped_matmul_int32(rows_q, lay.w1_t, counts)
+    hq, hs = O.dequant_swiglu_quant(acc1, lay.s13, rows_s, counts)
+    grp = torch.repeat_interleave(torch.arange(5), counts)
+    exact2 = torch.stack([hq[m].double() @ lay.w2_t[grp[m]].double() for m in range(M)])
+    want = (exact2 * s2_used.double()[grp] * hs.double().unsqueeze(1)).to(torch.bfloat16)
+    other = (exact2 * s2_other.double()[grp] * hs.double().unsqueeze(1)).to(torch.bfloat16)
+    steps = _bf16_steps(got, want)
+    assert int(steps.max()) <= 1 and float((steps == 0).float().mean()) > 0.99
+    assert float((_bf16_steps(got, other) == 0).float().mean()) < 0.9, "the other scale precision is not distinguishable"
+    # (c) shifted group boundaries give another result
+    shifted = torch.tensor([10, 0, 22, 1, 14])
+    wit_shift, _ = _fp64_expert_rows(rows_q, rows_s, lay.w1_t, lay.s13, lay.w2_t, s2_used, shifted)
+    assert rel_err(got.float(), wit_shift) > 0.05
+
+
+def _fp64_shared(x, w_gate_up, s_gate_up, w_down, s_down):
+    """The shared expert on the W8A8 scheme in float64 (quantisation steps included)."""
+    xf = x.double()
+    s = xf.abs().amax(1) / 127.0
+    q = torch.round(xf / s.unsqueeze(1)).clamp(-128, 127)
+    d = (q @ w_gate_up.double()) * s_gate_up.double() * s.unsqueeze(1)
+    inter = d.shape[1] // 2
+    y = d[:, :inter] / (1 + torch.exp(-d[:, :inter])) * d[:, inter:]
+    s2 = y.abs().amax(1) / 127.0
+    q2 = torch.round(y / s2.unsqueeze(1)).clamp(-128, 127)
+    return (q2 @ w_down.double()) * s_down.double() * s2.unsqueeze(1)
+
+
+def test_deepseek_moe_forward_against_fp64_witness():
+    """DeepseekMoE._forward_*_norm without collectives (deepseek_moe.py:243-368).
+    (a) whole block against a permutation-free fp64 witness: library router (transformers) for the
+    selection, dense brute force for the routed experts, fp64 shared expert;  a wrong expert range or a
+    missing shared expert fails;  (b) the shared output is added as a bf16 tensor to the bf16 routed
+    output (deepseek_moe.py:303,366), not in fp32 before the rounding: the block with the shared expert
+    must equal bf16(block without + shared) bit for bit."""
+    E, n_local, K, ng, tg, H, I, T = 32, 4, 8, 8, 4, 512, 256, 96
+    lay = Layer(n_local, H, I, seed=33, shared=True)
+    g = gen(34)
+    x = tokens(T, H, 34)
+    logits = torch.randn(T, E, generator=g) * 2
+    logits[:, 8:12] += 2.0                      # make the local experts (ids 8..11) popular
+    bias = torch.randn(E, generator=g) * 0.01
+    lo = 8
+    routed = (lay.w1_t, lay.s13, lay.w2_t, lay.s2)
+    out, st = O.deepseek_moe_forward(x, logits, bias, routed, lay.shared, K, ng, tg, 2.5, (lo, lo + n_local),
+                                     return_stages=True)
+    assert out.dtype == torch.bfloat16
+    # (a) independent selection and weights from the library router
+    with torch.no_grad():
+        _, hw, hi = _hf_router(E, K, ng, tg, 2.5, bias)(logits)
+    xq, xs = O.dynamic_quant(x)
+    dense_routed = O.dense_bruteforce(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, hw, hi.int(), (lo, lo + n_local))
+    assert int(((hi >= lo) & (hi < lo + n_local)).sum()) > T     # the local range really is exercised
+    wit = dense_routed + _fp64_shared(x, *lay.shared)
+    assert rel_err(out.float(), wit) < 6e-3 and cosine(out.float(), wit) > 0.9999
+    wrong_range = O.dense_bruteforce(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, hw, hi.int(), (lo + 1, lo + 1 + n_local))
+    assert rel_err(out.float(), wrong_range + _fp64_shared(x, *lay.shared)) > 0.05
+    assert rel_err(out.float(), dense_routed) > 0.05               # the shared expert is in the sum
+    # (b) rounding points of the final add
+    out_wo = O.deepseek_moe_forward(x, logits, bias, routed, None, K, ng, tg, 2.5, (lo, lo + n_local))
+    sh = O.shared_expert_mlp(x, *lay.shared)
+    assert out_wo.dtype == torch.bfloat16 and sh.dtype == torch.bfloat16
+    assert torch.equal(out, out_wo + sh)
+    fp32_add = (st["out32"] + _fp64_shared(x, *lay.shared).float()).to(torch.bfloat16)
+    assert not torch.equal(out, fp32_add)                          # and that is a different number
