@@ -234,6 +234,25 @@ int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, con
                         size_t ws_bytes, void* stream);
 size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared, int rows_dtype);
 
+/*
+ * The same layer on the library's own scratch.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory or hold a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  Arguments and results are those of omni_moe_w8a8_layer
+ * without the workspace; the scratch is a static device array of OMNI_STATIC_SCRATCH_BYTES that every
+ * GPU the library runs on holds until the process ends.  A call that would need more scratch (at the
+ * DeepSeek-V3 shape with 32 local experts, a shared expert and fp32 rows: more than about 128 tokens, and
+ * any shape whose row counts select the large-tile GEMM kernel) is refused with OMNI_E_WORKSPACE.
+ * The call allocates nothing and frees nothing.  Its first call on a device looks up that device's copy
+ * of the array (make that call outside a stream capture).  All calls on one GPU share the array, so two
+ * calls that overlap in time on one GPU (different streams) race; calls on one stream are safe.
+ */
+#define OMNI_STATIC_SCRATCH_BYTES 67108864 /* 64 MiB */
+int omni_moe_w8a8_layer_static(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
+                               const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
+                               const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
+                               const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
+                               const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,6 +33,7 @@ SIGNATURES = {
     "omni_moe_combine": (I, [P, I, P, P, I, I, I, I, I, P, P, P, P, P]),
     "omni_moe_w8a8_layer": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
     "omni_moe_w8a8_layer_workspace_bytes": (c_size_t, [I, I, I, I, I, I, I]),
+    "omni_moe_w8a8_layer_static": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, I, P, P]),
 }
 
 OMNI_DT_BF16, OMNI_DT_F32, OMNI_DT_F16 = 0, 1, 2
@@ -42,6 +43,7 @@ OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_REQUANT = 1, 4
 OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 
+OMNI_STATIC_SCRATCH_BYTES = 64 << 20
 ABI_VERSION = 3   # omni_moe_abi_version() of the header these signatures were written from
 
 _lib = None

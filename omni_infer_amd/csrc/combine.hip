@@ -7,6 +7,8 @@
 
 #include <string.h>
 
+#include <mutex>
+
 // ---------------------------------------------------------------- error state
 static thread_local char g_err[512] = "";
 void omni_set_error(const char* fmt, ...) {
@@ -287,4 +289,57 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
   return omni_moe_combine(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
                           nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,
                           stream);
+}
+
+// ---------------------------------------------------------------- whole layer on the library's own scratch
+// The same layer for callers that must not allocate and have no workspace to pass (code under HIP graph
+// capture, tight serving loops).  The scratch is a file-scope device array: every GPU the library runs on
+// holds one copy of it, at an address of its own, until the process ends.  The array's name is only a
+// host-side handle; the device address is asked for once per device and used from then on.
+namespace {
+static __device__ __align__(256) unsigned char scratch[OMNI_STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_ptr[MAX_DEVICES];
+std::mutex g_scratch_mutex;
+
+// device address of this device's copy of `scratch` (resolved on the first call with that device current)
+int static_scratch_ptr(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    OMNI_FAIL(OMNI_E_LAUNCH, "layer_static: no current device (or device index >= %d)", MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      OMNI_FAIL(OMNI_E_LAUNCH, "layer_static: hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return OMNI_OK;
+}
+}  // namespace
+
+extern "C" int omni_moe_w8a8_layer_static(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
+                                          const int32_t* topk_ids, int T, int K, int lo, int hi,
+                                          const int8_t* w13_packed, const float* w13_scale, const int8_t* w2_packed,
+                                          const float* w2_scale, const int8_t* sh13_packed, const float* sh13_scale,
+                                          const int8_t* sh2_packed, const float* sh2_scale, int H, int I,
+                                          int rows_dtype, void* out_bf16, void* stream) {
+  if (T < 0 || K <= 0 || hi <= lo || H <= 0 || I <= 0) OMNI_FAIL(OMNI_E_INVALID, "layer_static: bad sizes");
+  if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "layer_static: rows_dtype %d", rows_dtype);
+  const size_t need = layer_layout(T, K, hi - lo, H, I, sh13_packed != nullptr, rows_dtype).total;
+  if (need > (size_t)OMNI_STATIC_SCRATCH_BYTES)
+    OMNI_FAIL(OMNI_E_WORKSPACE,
+              "layer_static: this call needs %zu bytes of scratch, the library's static scratch holds %zu; "
+              "use omni_moe_w8a8_layer with a workspace for calls of this size",
+              need, (size_t)OMNI_STATIC_SCRATCH_BYTES);
+  void* ptr = nullptr;
+  const int rc = static_scratch_ptr(&ptr);
+  if (rc) return rc;
+  // nothing in the scratch has to start at zero except the arrival counters of split tiles, and the tile
+  // launch clears those itself with a fill kernel; everything else is written before it is read
+  return omni_moe_w8a8_layer(x, x_dtype, x_scale_in, topk_w, topk_ids, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
+                             w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, ptr,
+                             (size_t)OMNI_STATIC_SCRATCH_BYTES, stream);
 }

@@ -349,3 +349,30 @@ def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: tor
     L.check(rc, "omni_moe_w8a8_layer")
     return out
 
+
+def moe_w8a8_layer_static(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: torch.Tensor, topk_ids: torch.Tensor,
+                          lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None, H: int = 0,
+                          I: int = 0, out: Optional[torch.Tensor] = None,
+                          rows_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``moe_w8a8_layer`` on the library's static scratch: the call allocates nothing on the device
+    when ``out`` is given and the inputs are already fp32 / int32 / contiguous.  Sizes that need more
+    than ``OMNI_STATIC_SCRATCH_BYTES`` of scratch raise RuntimeError.  Calls that overlap in time on
+    one GPU share the scratch and race; calls on one stream are safe."""
+    _need_gpu(x, topk_w, topk_ids)
+    T, K = topk_ids.shape
+    if not (x.is_contiguous() and topk_w.is_contiguous() and topk_ids.is_contiguous() and
+            topk_w.dtype == torch.float32 and topk_ids.dtype == torch.int32):
+        raise ValueError("moe_w8a8_layer_static: contiguous inputs, fp32 weights and int32 ids only (no conversion "
+                         "copies are made here)")
+    if rows_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("rows_dtype must be torch.float32 or torch.bfloat16")
+    x_dtype = -1 if x.dtype == torch.int8 else _DT[x.dtype]
+    sh = shared if shared is not None else (None, None, None, None)
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
+    rc = L.lib().omni_moe_w8a8_layer_static(_ptr(x), x_dtype, _ptr(x_scale), _ptr(topk_w), _ptr(topk_ids), T, K, lo, hi,
+                                            _ptr(w13_packed), _ptr(w13_scale), _ptr(w2_packed), _ptr(w2_scale),
+                                            _ptr(sh[0]), _ptr(sh[1]), _ptr(sh[2]), _ptr(sh[3]), H, I, _DT[rows_dtype],
+                                            _ptr(out), _stream())
+    L.check(rc, "omni_moe_w8a8_layer_static")
+    return out
