@@ -93,6 +93,25 @@ int omni_moe_route(const float* logits, const float* bias, int T, int E, int n_g
                    float eps, float* topk_w, int32_t* topk_ids, void* stream);
 
 /*
+ * Gate projection + router in two launches.  Replaces self.gate.forward(hidden_states.float()) followed by
+ * FusedMoE.select_experts (omni/models/common/layers/moe/deepseek_moe.py:147-152,253-256,329; the bf16 gate
+ * of omni/models/deepseek/deepseek_v3_a2.py:607-613 with w_dtype BF16 and round_logits_bf16 = 1).
+ *   x [T,H] bf16 or fp32 (x_dtype), gate_w [E,H] fp32 or bf16 (w_dtype), H % 128 == 0, E <= 512.
+ *   logits[t][e] = sum_k x[t][k] * gate_w[e][k] on the fp32 matrix cores in a fixed order: the reduction is cut
+ *   into slices of 128 elements, each summed as a chain of fused multiply-adds over ascending k starting from
+ *   +0 (v_mfma_f32_32x32x1_2b_f32 is one fma per output element); 8 consecutive slices are added left to right
+ *   into a group sum, and the group sums left to right into the logit.  The result does not depend on T.
+ *   The logits are then routed exactly as omni_moe_route routes them (same arguments); they are written to
+ *   logits_out when it is not NULL; K = 0 computes the logits only (topk_* may be NULL).
+ *   workspace: omni_moe_gate_route_workspace_bytes(T, H, E) (partial sums), 16-byte aligned.
+ */
+int omni_moe_gate_route(const void* x, int x_dtype, const void* gate_w, int w_dtype, const float* bias, int T, int H,
+                        int E, int n_group, int topk_group, int K, int score_fn, int group_mode, int masked_fill_zero,
+                        int weight_from_c, int renorm, float scale, float eps, int round_logits_bf16, float* logits_out,
+                        float* topk_w, int32_t* topk_ids, void* workspace, size_t ws_bytes, void* stream);
+size_t omni_moe_gate_route_workspace_bytes(int T, int H, int E);
+
+/*
  * Per-row dynamic int8 quantisation.  Replaces torch_npu.npu_dynamic_quant
  * (omni/models/common/layers/moe/deepseek_moe.py:247,323,612;
  * omni/quantization/compressed_tensors/compressed_tensors_moe.py:241,247;

@@ -19,6 +19,8 @@ SIGNATURES = {
     "omni_moe_last_error": (c_char_p, []),
     "omni_moe_abi_version": (I, []),
     "omni_moe_route": (I, [P, P, I, I, I, I, I, I, I, I, I, I, c_float, c_float, P, P, P]),
+    "omni_moe_gate_route": (I, [P, I, P, I, P, I, I, I, I, I, I, I, I, I, I, I, c_float, c_float, I, P, P, P, P, c_size_t, P]),
+    "omni_moe_gate_route_workspace_bytes": (c_size_t, [I, I, I]),
     "omni_dynamic_quant": (I, [P, I, c_int64, I, c_int64, P, P, P]),
     "omni_add_rms_norm_quant": (I, [P, P, P, c_int64, I, c_float, P, P, P, P, P]),
     "omni_moe_permute": (I, [P, I, I, I, I, I, P, P, P, P, P, c_size_t, P]),

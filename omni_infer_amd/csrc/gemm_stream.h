@@ -1,0 +1,340 @@
+// The weight-streaming grouped int8 GEMM block (decode-sized batches) and what it shares with the other
+// GEMM kernels: the argument record, the source-row lookup and the GEMM2 row epilogue.
+#pragma once
+#include "common.h"
+
+namespace {
+
+struct GemmArgs {
+  const int8_t* a_q;        // GEMM1: [T, Kdim] source rows; GEMM2: [M_cap, Kdim] sorted rows
+  const float* a_scale;     // per source row (GEMM1) / per sorted row (GEMM2)
+  const int32_t* sorted_src;  // GEMM1 only, nullable
+  int idx_mode, T, K;
+  const int8_t* w;
+  const float* w_scale;
+  const int8_t* w_extra;
+  const float* w_extra_scale;
+  int extra_rows;
+  const int32_t* offsets;
+  int G;
+  int Kdim;  // reduction length
+  int N;     // output channels of the GEMM: 2I (GEMM1) or H (GEMM2)
+  int flags;
+  float* y;            // GEMM1: [M_cap, I]
+  void* rows_out;      // GEMM2: [M_cap, N]
+  int out_dtype;
+  int32_t* acc_dbg;    // [M_cap, N], nullable
+  int tile_gx, tile_gy, tile_pc;  // tile kernel: column tiles, row blocks (worst case), columns of a patch
+  int tile_slots;                 // tile kernel: blocks the chip runs at once
+  int tile_split_max;             // tile kernel: most shares a tile of the last partial round is split into
+  int32_t* tail_cnt;              // tile kernel: arrival counters of the split tiles (zero at launch), or null
+  int32_t* tail_part;             // tile kernel: partial accumulators of the split tiles
+  int32_t* part;       // GEMM1 stream kernel: [S, M_cap, N] partial accumulators (split-k)
+  int S;               // number of k splits (grid.z)
+  int64_t M_cap;
+};
+
+// source row of sorted row r of group g
+template <int KIND>
+__device__ __forceinline__ int source_row(const GemmArgs& a, int g, int r) {
+  if constexpr (KIND == 2) {
+    return r;
+  } else {
+    if (g >= a.G) return r - a.offsets[a.G];
+    if (a.sorted_src == nullptr) return r;
+    int s = a.sorted_src[r];
+    return (a.idx_mode == OMNI_IDX_TOKEN_MAJOR) ? s / a.K : s % a.T;
+  }
+}
+
+__device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float* __restrict__ wsc, int n, int row0,
+                                               int rbase, int nrows, const float* ts, v4i acc) {
+  const float ws = wsc[n];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int rr = rbase + i;
+    if (rr < nrows) {
+      float o = ((float)acc[i] * ws) * ts[i];
+      size_t m = (size_t)(row0 + rr);
+      if (a.out_dtype == OMNI_DT_F32) ((float*)a.rows_out)[m * (size_t)a.N + n] = o;
+      else ((uint16_t*)a.rows_out)[m * (size_t)a.N + n] = f32_to_bf16(o);
+      if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + n] = acc[i];
+    }
+  }
+}
+
+// =====================================================================================
+// gemm_stream
+//   KIND 1: a wavefront owns NT (gate, up) strip pairs; KIND 2: NT strips.
+//   MT: 16-row tiles per block (block covers up to 16*MT rows of one group).
+//   D : k-steps of B kept in flight per wavefront (multiple of 4).
+//   Requires Kdim % (64*D) == 0 (checked on the host).
+//
+// The k loop is free of data-dependent branches: rows past the end of a group read the group's
+// first row (their accumulators are never stored), every tile of the block is multiplied, and
+// the loop is split into a part that refills the ring and a drain part, so the compiler can
+// count outstanding loads exactly and never waits for more than the oldest k-step.
+// =====================================================================================
+// Occupancy asked of the compiler: the small variants are held to 5 wavefronts per SIMD (96
+// registers) so that a decode-sized launch (about 34 row blocks x 32 channel blocks) is resident
+// all at once: a second, nearly empty round of blocks would stream at a fraction of the bandwidth.
+template <int KIND, int MT, int NT, int D>
+constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1; }
+
+// One block's work: the rows of row block `rb` times the channels of column block `bx` (4 wavefronts x NT
+// strips, or strip pairs), k share `bz` of a.S.  `before_a()` runs after the first D k-steps of B have been
+// requested and before anything of A is touched: a caller whose A is still being produced waits there,
+// with its weight loads already in flight.  All four wavefronts of the block must call this together
+// (block barriers inside); when it returns nobody reads the LDS buffers any more.
+template <int KIND, int MT, int NT, int D, typename BeforeA>
+__device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& rb, int bx, int bz,
+                                             v4i (*lds_a)[MT * 4 * WAVE], BeforeA before_a) {
+  constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
+  constexpr int DC = D / 4;                       // chunks (4 k-steps) of B in flight
+  static_assert(D % 4 == 0, "D counts whole chunks");
+
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int w = threadIdx.x / WAVE;
+  const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
+  const int mt_cnt = (nrows + 15) / 16;
+  const int nk64_all = a.Kdim / 64;          // k-steps of the whole reduction
+  const int nk64 = nk64_all / a.S;           // k-steps of this block's share
+  const int k64_0 = bz * nk64;
+  const int nchunks = nk64 / 4;
+  const int I = (KIND == 1) ? a.N / 2 : 0;
+
+  const int8_t* wbase = (g < a.G) ? a.w + (size_t)g * a.Kdim * a.N : a.w_extra;
+  const float* wsc = (g < a.G) ? a.w_scale + (size_t)g * a.N : a.w_extra_scale;
+
+  // strips of this wavefront
+  int strip[NBF];
+  const int8_t* bp[NBF];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int q = (bx * 4 + w) * NT + t;
+    if constexpr (KIND == 1) {
+      strip[2 * t] = q;
+      strip[2 * t + 1] = I / 16 + q;
+    } else {
+      strip[t] = q;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NBF; ++j) bp[j] = wbase + ((size_t)strip[j] * nk64_all + k64_0) * 1024 + lane * 16;
+
+  // the first D k-steps of B are requested as soon as their addresses exist (they come from HBM and
+  // take the longest); the A row lookup below overlaps with their flight
+  v4i ring[D][NBF];
+#pragma unroll
+  for (int s = 0; s < D; ++s)
+#pragma unroll
+    for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
+  __builtin_amdgcn_sched_barrier(0);
+  before_a();
+
+  // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile, k-step w of
+  // every chunk; rows past the end of the group alias the group's first row
+  const int8_t* arow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int rr = mt * 16 + (lane & 15);
+    if (rr >= nrows) rr = 0;
+    arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k64_0 * 64 + (lane >> 4) * 16 + w * 64;
+  }
+
+  v4i acc[MT][NBF];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < NBF; ++j) acc[mt][j] = (v4i){0, 0, 0, 0};
+
+  // ---- prologue: A chunk 0 -> LDS
+  v4i areg[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt]);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) lds_a[0][(mt * 4 + w) * WAVE + lane] = areg[mt];
+  __syncthreads();
+
+  // one chunk = 4 k-steps on ring slots [4*cc, 4*cc+4)
+  auto chunk = [&](const int c, const int cc, const bool refill) {
+    const int cnext = (c + 1 < nchunks) ? c + 1 : c;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt] + (size_t)cnext * 256);
+    // keep these loads ahead of the ring refills below: they are waited for at the end of the
+    // chunk, and loads complete in order, so a later position would drain the whole ring
+    __builtin_amdgcn_sched_barrier(0);
+    const v4i* la = lds_a[c & 1];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int s = cc * 4 + kk;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        v4i af = la[(mt * 4 + kk) * WAVE + lane];
+#pragma unroll
+        for (int j = 0; j < NBF; ++j) acc[mt][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, ring[s][j], acc[mt][j], 0, 0, 0);
+      }
+      // the slot is free once its MFMAs are issued: refill it with the k-step D ahead
+      if (refill) {
+#pragma unroll
+        for (int j = 0; j < NBF; ++j)
+          ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)(c * 4 + kk + D) * 1024));
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one k-step at a time: refills stay spread over the chunk
+    }
+    v4i* ln = lds_a[(c + 1) & 1];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) ln[(mt * 4 + w) * WAVE + lane] = areg[mt];
+    __syncthreads();
+  };
+
+  int c0 = 0;
+  for (; c0 < nchunks - DC; c0 += DC) {
+#pragma unroll
+    for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, true);
+  }
+#pragma unroll
+  for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, false);
+
+  // ---- epilogue
+  const int col = lane & 15;
+  if constexpr (KIND == 1) {
+    if (a.y != nullptr) {
+      // a single k share: the wavefront holds the gate and the up sums of its channels, so it
+      // dequantises and applies SwiGLU here; the row quantiser is left with the maximum and the rounding
+      const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if (mt < mt_cnt) {
+          const int rbase = mt * 16 + 4 * (lane >> 4);
+          float ts[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            ts[i] = (rbase + i < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rbase + i)] : 0.0f;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const int n = strip[2 * t] * 16 + col;
+            const float wg = wsc[n], wu = wsc[I + n];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (rbase + i < nrows) {
+                float dg = ((float)acc[mt][2 * t][i] * wg) * ts[i];
+                float du = ((float)acc[mt][2 * t + 1][i] * wu) * ts[i];
+                if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
+                float yv = silu_spec(dg) * du;
+                if (bf) yv = round_bf16(yv);
+                a.y[(size_t)(row0 + rbase + i) * I + n] = yv;
+              }
+            }
+          }
+        }
+      }
+      return;
+    }
+    // raw int32 partial sums of this k share; the row kernel adds the shares and finishes
+    int32_t* part = a.part + (size_t)bz * a.M_cap * a.N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (mt < mt_cnt) {
+        const int rbase = mt * 16 + 4 * (lane >> 4);
+#pragma unroll
+        for (int j = 0; j < NBF; ++j) {
+          const int n = strip[j] * 16 + col;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (rbase + i < nrows) part[(size_t)(row0 + rbase + i) * a.N + n] = acc[mt][j][i];
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (mt < mt_cnt) {
+        const int rbase = mt * 16 + 4 * (lane >> 4);
+        float ts[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int rr = rbase + i;
+          ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsc, strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
+      }
+    }
+  }
+}
+
+template <int KIND, int MT, int NT, int D>
+__global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void gemm_stream(GemmArgs a) {
+  __shared__ v4i lds_a[2][MT * 4 * WAVE];
+  RowBlock rb;
+  if (!find_row_block(a.offsets, a.G, a.extra_rows, 16 * MT, blockIdx.y, rb)) return;
+  stream_block<KIND, MT, NT, D>(a, rb, blockIdx.x, blockIdx.z, lds_a, [] {});
+}
+
+// Row quantisation of y = silu(gate) * up (fp32) by one wavefront: scale = max|y| / 127, q = rint(y / scale).
+// Up to 256*NV values are kept in registers between the maximum and the rounding, so the row is read
+// once; NV == 0 reads it twice.  The two halves are separate so that a caller can have the loads of
+// several rows in flight before it reduces the first.
+template <int NV>
+__device__ __forceinline__ void load_row_y(const float* __restrict__ yr, int I, int lane, v4f (&v)[NV]) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (i * WAVE + lane) * 4;
+    v[i] = (c < I) ? __builtin_nontemporal_load((const v4f*)(yr + c)) : (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+  }
+}
+template <int NV>
+__device__ __forceinline__ void quant_loaded_row(const v4f (&v)[NV], int I, int8_t* __restrict__ qr,
+                                                 float* __restrict__ hs_m, int lane) {
+  float mx = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(v[i][j]));
+  mx = wave_allmax_f(mx);
+  const float s = mx / 127.0f;
+  if (lane == 0) *hs_m = s;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = (i * WAVE + lane) * 4;
+    if (c < I) {
+      uint32_t o = 0;
+      if (s > 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o |= ((uint32_t)(quant_i8(v[i][j], s) & 0xff)) << (8 * j);
+      }
+      *(uint32_t*)(qr + c) = o;
+    }
+  }
+}
+template <int NV>
+__device__ __forceinline__ void quant_row_y_wave(const float* __restrict__ yr, int I, int8_t* __restrict__ qr,
+                                                 float* __restrict__ hs_m, int lane) {
+  if constexpr (NV > 0) {
+    v4f v[NV];
+    load_row_y<NV>(yr, I, lane, v);
+    quant_loaded_row<NV>(v, I, qr, hs_m, lane);
+  } else {
+    float mx = 0.0f;
+    for (int c = lane * 4; c < I; c += WAVE * 4) {
+      v4f v = *(const v4f*)(yr + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mx = fmaxf(mx, fabsf(v[j]));
+    }
+    mx = wave_allmax_f(mx);
+    const float s = mx / 127.0f;
+    if (lane == 0) *hs_m = s;
+    for (int c = lane * 4; c < I; c += WAVE * 4) {
+      v4f v = *(const v4f*)(yr + c);
+      uint32_t o = 0;
+      if (s > 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o |= ((uint32_t)(quant_i8(v[j], s) & 0xff)) << (8 * j);
+      }
+      *(uint32_t*)(qr + c) = o;
+    }
+  }
+}
+
+}  // namespace

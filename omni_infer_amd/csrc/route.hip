@@ -4,12 +4,37 @@
 // the K selection rounds are all wave-level reductions (DPP inside a row of 16 lanes, bpermute
 // across rows); nothing goes through LDS or global memory between the logits load and the
 // K (weight, id) stores.
+//
+// The same kernel also finishes the gate projection: when it is given partial sums of the logits
+// (gate_partial_kernel below) it adds them up in the stated order before it routes, so the logits
+// never make a round trip of their own and the two launches of this file are the whole
+// gate + router.
+//
+// Gate projection: logits[t][e] = sum_k x[t][k] * w[e][k] on the fp32 matrix cores with a fixed order.
+//   v_mfma_f32_32x32x1_2b_f32 is a rank-1 update, one fused multiply-add (a single rounding) per
+//   output element; a run of them over ascending k is therefore an exactly specified chain
+//       acc = fma(x[t][k], w[e][k], acc),  acc = +0 at the start of a slice.
+//   The reduction is cut into slices of 128 elements and groups of 8 slices:
+//       P_s = fma chain over slice s;  Q_g = P_8g + P_8g+1 + ... (left to right, fp32 adds);
+//       logits = Q_0 + Q_1 + ... (left to right).
+//   How the slices are dealt to wavefronts (one slice each for small batches, one group each for
+//   large ones) does not change a bit of the result.
 #include "common.h"
 
 namespace {
 
+constexpr int GATE_SLICE = 128;  // reduction elements of one fma chain
+constexpr int GATE_GROUP = 8;    // slices added up before the groups are
+
 struct RouteArgs {
   const float* logits;
+  // partial sums of the logits instead of the logits: [n_parts][T][E]; parts are slices (group_len 8) or
+  // whole groups (group_len 1)
+  const float* partials;
+  int n_parts, group_len;
+  int fold_block;        // the four wavefronts of a block add up one token's parts together
+  float* logits_out;     // nullable: the finished logits
+  int round_logits_bf16; // round the finished logits to bf16 (the bf16 gate of deepseek_v3_a2.py:607-613)
   const float* bias;
   int T, E, n_group, topk_group, K;
   int score_fn, group_mode, masked_fill_zero, weight_from_c, renorm;
@@ -20,21 +45,94 @@ struct RouteArgs {
 
 constexpr float NEG_INF = -__builtin_inff();
 
+constexpr int FOLD_MAX_GROUPS = 16;  // groups of partial sums the block-wide fold takes (H <= 16384)
+
 template <int V>
 __global__ __launch_bounds__(256) void route_kernel(RouteArgs a) {
   const int lane = threadIdx.x & (WAVE - 1);
-  const int t = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
+  const int wv = threadIdx.x / WAVE;
+  // one token per wavefront; with fold_block one token per block: its four wavefronts add up the partial
+  // sums of the gate projection together (one round of loads), then the first one routes
+  const int t = a.fold_block ? (int)blockIdx.x : (int)blockIdx.x * (blockDim.x / WAVE) + wv;
   if (t >= a.T) return;  // whole wave leaves together
-  const float* row = a.logits + (size_t)t * a.E;
 
   float s[V];  // score
   float c[V];  // selection score
   bool in[V];
 #pragma unroll
-  for (int j = 0; j < V; ++j) {
-    int e = lane * V + j;
-    in[j] = e < a.E;
-    s[j] = in[j] ? row[e] : NEG_INF;
+  for (int j = 0; j < V; ++j) in[j] = lane * V + j < a.E;
+  if (a.partials == nullptr) {
+    const float* row = a.logits + (size_t)t * a.E;
+#pragma unroll
+    for (int j = 0; j < V; ++j) s[j] = in[j] ? row[lane * V + j] : NEG_INF;
+  } else {
+    // finish the gate projection: groups of `group_len` parts left to right, then the groups left to right
+    const size_t plane = (size_t)a.T * a.E;
+    const float* p0 = a.partials + (size_t)t * a.E + lane * V;
+    const int n_groups = (a.n_parts + a.group_len - 1) / a.group_len;
+    // sum of group g: its parts are all requested before the first add
+    auto load_group = [&](int g, float (&part)[GATE_GROUP][V]) {
+      const int g0 = g * a.group_len;
+      const int gl = (g < n_groups) ? min(a.group_len, a.n_parts - g0) : 0;
+#pragma unroll
+      for (int u = 0; u < GATE_GROUP; ++u)
+#pragma unroll
+        for (int j = 0; j < V; ++j) part[u][j] = (u < gl && in[j]) ? p0[(size_t)(g0 + u) * plane + j] : 0.0f;
+      return gl;
+    };
+    auto fold_group = [&](const float (&part)[GATE_GROUP][V], int gl, float (&q)[V]) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) q[j] = part[0][j];
+#pragma unroll
+      for (int u = 1; u < GATE_GROUP; ++u)
+        if (u < gl) {
+#pragma unroll
+          for (int j = 0; j < V; ++j) q[j] = q[j] + part[u][j];
+        }
+    };
+    float tot[V];
+    if (a.fold_block) {
+      __shared__ float s_q[FOLD_MAX_GROUPS][WAVE * V];
+      // wavefront wv takes groups wv, wv + 4, ...: two of them are loaded before either is added up
+      for (int base = 0; base < n_groups; base += 8) {
+        float pa[GATE_GROUP][V], pb[GATE_GROUP][V], q[V];
+        const int ga = base + wv, gb = base + 4 + wv;
+        const int la = load_group(ga, pa);
+        const int lb = load_group(gb, pb);
+        if (la > 0) {
+          fold_group(pa, la, q);
+#pragma unroll
+          for (int j = 0; j < V; ++j) s_q[ga][lane * V + j] = q[j];
+        }
+        if (lb > 0) {
+          fold_group(pb, lb, q);
+#pragma unroll
+          for (int j = 0; j < V; ++j) s_q[gb][lane * V + j] = q[j];
+        }
+      }
+      __syncthreads();
+      if (wv != 0) return;
+#pragma unroll
+      for (int j = 0; j < V; ++j) tot[j] = s_q[0][lane * V + j];
+      for (int g = 1; g < n_groups; ++g)
+#pragma unroll
+        for (int j = 0; j < V; ++j) tot[j] = tot[j] + s_q[g][lane * V + j];
+    } else {
+      for (int g = 0; g < n_groups; ++g) {
+        float part[GATE_GROUP][V], q[V];
+        const int gl = load_group(g, part);
+        fold_group(part, gl, q);
+#pragma unroll
+        for (int j = 0; j < V; ++j) tot[j] = (g == 0) ? q[j] : tot[j] + q[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      if (a.round_logits_bf16) tot[j] = round_bf16(tot[j]);
+      s[j] = in[j] ? tot[j] : NEG_INF;
+      if (a.logits_out != nullptr && in[j]) a.logits_out[(size_t)t * a.E + lane * V + j] = tot[j];
+    }
+    if (a.K == 0) return;  // the logits were all that was asked for
   }
   if (a.score_fn == OMNI_SCORE_SIGMOID) {
 #pragma unroll
@@ -167,6 +265,139 @@ __global__ __launch_bounds__(256) void route_kernel(RouteArgs a) {
   }
 }
 
+
+// ---------------------------------------------------------------- gate projection, partial sums
+struct GateArgs {
+  const void* x;   // [T, H] bf16 or fp32
+  const void* w;   // [E, H] fp32 or bf16
+  int T, H, E;
+  int slices_per_task;  // 1 or GATE_GROUP
+  int n_parts;          // H / 128 / slices_per_task, rounded up
+  int n_tt, n_et;       // token tiles of 64, expert tiles of 32
+  float* partials;      // [n_parts][T][E]
+};
+
+typedef float v32f __attribute__((ext_vector_type(32)));
+
+// 32 consecutive reduction elements of one row as floats, loaded with 16-byte loads
+template <int DT>
+struct Chunk32;
+template <>
+struct Chunk32<OMNI_DT_F32> {
+  v4f r[8];
+  __device__ __forceinline__ void load(const void* row, int k) {
+    const v4f* p = (const v4f*)((const float*)row + k);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = p[i];
+  }
+  __device__ __forceinline__ float at(int k) const { return r[k >> 2][k & 3]; }
+};
+template <>
+struct Chunk32<OMNI_DT_BF16> {
+  v4i r[4];
+  __device__ __forceinline__ void load(const void* row, int k) {
+    const v4i* p = (const v4i*)((const uint16_t*)row + k);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = p[i];
+  }
+  __device__ __forceinline__ float at(int k) const {
+    const uint32_t word = (uint32_t)r[k >> 3][(k >> 1) & 3];
+    return __uint_as_float((k & 1) ? (word & 0xffff0000u) : (word << 16));
+  }
+};
+
+// One wavefront per task: 64 tokens x 32 experts x `slices_per_task` slices of 128 reduction elements.
+// Lane l supplies token t0 + l (the matrix instruction's two 32-row blocks are the two halves of the token
+// tile) and expert e0 + l % 32.  The whole first slice is requested before the first multiply; while a chunk
+// of 32 elements is multiplied, the same chunk of the next slice is requested into the registers just used,
+// so the loads run a full slice (128 matrix instructions) ahead and one wavefront per SIMD keeps the matrix
+// pipe fed.  Output element (token t0 + 32 b + 8 (j/4) + 4 (l/32) + j%4, expert e0 + l%32) sits in
+// accumulator register 16 b + j of lane l.
+template <int XDT, int WDT>
+__global__ __launch_bounds__(64) void gate_partial_kernel(GateArgs a) {
+  const int lane = threadIdx.x;
+  int id = blockIdx.x;
+  const int tt = id % a.n_tt; id /= a.n_tt;
+  const int et = id % a.n_et; id /= a.n_et;
+  const int part = id;
+  const int n_slices = a.H / GATE_SLICE;
+  const int s_first = part * a.slices_per_task;
+  const int s_end = min(n_slices, s_first + a.slices_per_task);
+  const int tok = min(tt * 64 + lane, a.T - 1);           // rows past the end alias the last row; not stored
+  const int exp = min(et * 32 + (lane & 31), a.E - 1);
+  const size_t xes = (XDT == OMNI_DT_F32) ? 4 : 2, wes = (WDT == OMNI_DT_F32) ? 4 : 2;
+  const char* xrow = (const char*)a.x + (size_t)tok * a.H * xes;
+  const char* wrow = (const char*)a.w + (size_t)exp * a.H * wes;
+
+  Chunk32<XDT> xb[4];
+  Chunk32<WDT> wb[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    xb[c].load(xrow, s_first * GATE_SLICE + c * 32);
+    wb[c].load(wrow, s_first * GATE_SLICE + c * 32);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // the loads stay where they are written: ahead of the multiplies
+  v32f acc, q;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) { acc[i] = 0.0f; q[i] = 0.0f; }
+  for (int s = s_first; s < s_end; ++s) {
+    const int s_next = min(s + 1, s_end - 1);  // the last slice is requested once more instead of a branch
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+#pragma unroll
+      for (int k = 0; k < 32; ++k) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xb[c].at(k), wb[c].at(k), acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      xb[c].load(xrow, s_next * GATE_SLICE + c * 32);
+      wb[c].load(wrow, s_next * GATE_SLICE + c * 32);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // the slice's chain is complete: add it to the group's sum (the first slice starts it)
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      q[i] = (s == s_first) ? acc[i] : q[i] + acc[i];
+      acc[i] = 0.0f;
+    }
+  }
+  float* out = a.partials + (size_t)part * a.T * a.E;
+  const int e = et * 32 + (lane & 31);
+  if (e < a.E) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const int t = tt * 64 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * (lane >> 5) + (i & 3);
+      if (t < a.T) out[(size_t)t * a.E + e] = q[i];
+    }
+  }
+}
+
+// small batches: one slice per wavefront (many short tasks); large ones: a group of 8 slices each
+int gate_slices_per_task(int T, int H, int E) {
+  const int n_tt = (T + 63) / 64, n_et = (E + 31) / 32;
+  const int n_groups = (H / GATE_SLICE + GATE_GROUP - 1) / GATE_GROUP;
+  return ((int64_t)n_tt * n_et * n_groups >= 1024) ? GATE_GROUP : 1;
+}
+
+void launch_route(const RouteArgs& a, hipStream_t st) {
+  dim3 grid(a.fold_block ? a.T : (a.T + 3) / 4), block(256);
+  const int V = (a.E + 63) / 64;
+  if (V <= 1) hipLaunchKernelGGL(route_kernel<1>, grid, block, 0, st, a);
+  else if (V <= 2) hipLaunchKernelGGL(route_kernel<2>, grid, block, 0, st, a);
+  else if (V <= 4) hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, st, a);
+  else hipLaunchKernelGGL(route_kernel<8>, grid, block, 0, st, a);
+}
+
+int check_route_args(const char* what, int T, int E, int n_group, int topk_group, int K, int score_fn) {
+  if (E > 512) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: E=%d > 512", what, E);
+  if (K > 64 || K > E) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: K=%d must be <= min(64, E=%d)", what, K, E);
+  if (score_fn != OMNI_SCORE_SOFTMAX && score_fn != OMNI_SCORE_SIGMOID)
+    OMNI_FAIL(OMNI_E_INVALID, "%s: unknown score_fn %d", what, score_fn);
+  if (n_group > 1) {
+    if (n_group > 64 || E % n_group != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: n_group=%d must divide E=%d and be <= 64", what, n_group, E);
+    if (topk_group < 1 || topk_group > n_group) OMNI_FAIL(OMNI_E_INVALID, "%s: topk_group=%d out of range", what, topk_group);
+  }
+  (void)T;
+  return OMNI_OK;
+}
+
 }  // namespace
 
 extern "C" int omni_moe_route(const float* logits, const float* bias, int T, int E, int n_group, int topk_group,
@@ -175,23 +406,69 @@ extern "C" int omni_moe_route(const float* logits, const float* bias, int T, int
   if (T < 0 || E <= 0 || K <= 0) OMNI_FAIL(OMNI_E_INVALID, "route: bad sizes T=%d E=%d K=%d", T, E, K);
   if (T == 0) return OMNI_OK;
   if (!logits || !topk_w || !topk_ids) OMNI_FAIL(OMNI_E_INVALID, "route: null pointer");
-  if (E > 512) OMNI_FAIL(OMNI_E_UNSUPPORTED, "route: E=%d > 512", E);
-  if (K > 64 || K > E) OMNI_FAIL(OMNI_E_UNSUPPORTED, "route: K=%d must be <= min(64, E=%d)", K, E);
-  if (score_fn != OMNI_SCORE_SOFTMAX && score_fn != OMNI_SCORE_SIGMOID)
-    OMNI_FAIL(OMNI_E_INVALID, "route: unknown score_fn %d", score_fn);
-  if (n_group > 1) {
-    if (n_group > 64 || E % n_group != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "route: n_group=%d must divide E=%d and be <= 64", n_group, E);
-    if (topk_group < 1 || topk_group > n_group) OMNI_FAIL(OMNI_E_INVALID, "route: topk_group=%d out of range", topk_group);
-  }
-  RouteArgs a{logits, bias, T, E, n_group, topk_group, K, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm,
-              scale, eps, topk_w, topk_ids};
-  dim3 grid((T + 3) / 4), block(256);
-  hipStream_t st = (hipStream_t)stream;
-  int V = (E + 63) / 64;
-  if (V <= 1) hipLaunchKernelGGL(route_kernel<1>, grid, block, 0, st, a);
-  else if (V <= 2) hipLaunchKernelGGL(route_kernel<2>, grid, block, 0, st, a);
-  else if (V <= 4) hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, st, a);
-  else hipLaunchKernelGGL(route_kernel<8>, grid, block, 0, st, a);
+  const int rc = check_route_args("route", T, E, n_group, topk_group, K, score_fn);
+  if (rc) return rc;
+  RouteArgs a{logits, nullptr, 0, 1, 0, nullptr, 0, bias, T, E, n_group, topk_group, K, score_fn, group_mode, masked_fill_zero,
+              weight_from_c, renorm, scale, eps, topk_w, topk_ids};
+  launch_route(a, (hipStream_t)stream);
   OMNI_CHECK_LAUNCH("route");
+  return OMNI_OK;
+}
+
+extern "C" size_t omni_moe_gate_route_workspace_bytes(int T, int H, int E) {
+  if (T <= 0 || H <= 0 || E <= 0 || H % GATE_SLICE != 0) return 0;
+  const int spt = gate_slices_per_task(T, H, E);
+  const int n_parts = (H / GATE_SLICE + spt - 1) / spt;
+  return align256((size_t)n_parts * T * E * sizeof(float));
+}
+
+extern "C" int omni_moe_gate_route(const void* x, int x_dtype, const void* gate_w, int w_dtype, const float* bias, int T,
+                                   int H, int E, int n_group, int topk_group, int K, int score_fn, int group_mode,
+                                   int masked_fill_zero, int weight_from_c, int renorm, float scale, float eps,
+                                   int round_logits_bf16, float* logits_out, float* topk_w, int32_t* topk_ids,
+                                   void* workspace, size_t ws_bytes, void* stream) {
+  if (T < 0 || H <= 0 || E <= 0 || K < 0) OMNI_FAIL(OMNI_E_INVALID, "gate_route: bad sizes T=%d H=%d E=%d K=%d", T, H, E, K);
+  if (T == 0) return OMNI_OK;
+  if (!x || !gate_w) OMNI_FAIL(OMNI_E_INVALID, "gate_route: null pointer");
+  if (K == 0 && !logits_out) OMNI_FAIL(OMNI_E_INVALID, "gate_route: nothing to compute (K = 0 and no logits_out)");
+  if (K > 0 && (!topk_w || !topk_ids)) OMNI_FAIL(OMNI_E_INVALID, "gate_route: null pointer");
+  if ((x_dtype != OMNI_DT_BF16 && x_dtype != OMNI_DT_F32) || (w_dtype != OMNI_DT_BF16 && w_dtype != OMNI_DT_F32))
+    OMNI_FAIL(OMNI_E_INVALID, "gate_route: tokens and gate weights must be bf16 or fp32");
+  if (H % GATE_SLICE != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: H=%d must be a multiple of %d", H, GATE_SLICE);
+  if (((uintptr_t)x % 16) || ((uintptr_t)gate_w % 16)) OMNI_FAIL(OMNI_E_INVALID, "gate_route: pointers must be 16-byte aligned");
+  if (E > 512) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: E=%d > 512", E);
+  if (K > 0) {
+    const int rc = check_route_args("gate_route", T, E, n_group, topk_group, K, score_fn);
+    if (rc) return rc;
+  }
+  const size_t need = omni_moe_gate_route_workspace_bytes(T, H, E);
+  if (!workspace || ws_bytes < need) OMNI_FAIL(OMNI_E_WORKSPACE, "gate_route: workspace %zu < %zu", ws_bytes, need);
+  if ((uintptr_t)workspace % 16) OMNI_FAIL(OMNI_E_INVALID, "gate_route: workspace must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  GateArgs g{};
+  g.x = x; g.w = gate_w; g.T = T; g.H = H; g.E = E;
+  g.slices_per_task = gate_slices_per_task(T, H, E);
+  g.n_parts = (H / GATE_SLICE + g.slices_per_task - 1) / g.slices_per_task;
+  g.n_tt = (T + 63) / 64;
+  g.n_et = (E + 31) / 32;
+  g.partials = (float*)workspace;
+  const int64_t tasks = (int64_t)g.n_parts * g.n_et * g.n_tt;
+  if (tasks > 0x7fffffffLL) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: too many tasks");
+  dim3 grid((unsigned)tasks), block(64);
+  if (x_dtype == OMNI_DT_BF16 && w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_BF16, OMNI_DT_F32>), grid, block, 0, st, g);
+  else if (x_dtype == OMNI_DT_BF16) hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_BF16, OMNI_DT_BF16>), grid, block, 0, st, g);
+  else if (w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_F32, OMNI_DT_F32>), grid, block, 0, st, g);
+  else hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_F32, OMNI_DT_BF16>), grid, block, 0, st, g);
+  OMNI_CHECK_LAUNCH("gate_partial");
+  // few tokens: a block per token adds the parts up with its four wavefronts (the latency of one round of
+  // loads instead of one per group); many tokens: a wavefront per token keeps every wavefront routing
+  const int group_len = g.slices_per_task == 1 ? GATE_GROUP : 1;
+  const int n_groups = (g.n_parts + group_len - 1) / group_len;
+  const int fold_block = (T <= 2048 && n_groups <= FOLD_MAX_GROUPS) ? 1 : 0;
+  RouteArgs a{nullptr, g.partials, g.n_parts, group_len, fold_block, logits_out, round_logits_bf16, bias, T, E,
+              n_group, topk_group, K, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm, scale, eps, topk_w,
+              topk_ids};
+  launch_route(a, st);
+  OMNI_CHECK_LAUNCH("gate_route");
   return OMNI_OK;
 }

@@ -56,9 +56,72 @@ def moe_route(logits: torch.Tensor, bias: Optional[torch.Tensor], top_k: int, n_
     return w, ids
 
 
+_GATE_WS = {}
+
+
+def moe_gate_route(x: torch.Tensor, gate_w: torch.Tensor, bias: Optional[torch.Tensor], top_k: int, n_group: int,
+                   topk_group: int, score_fn: str, group_mode: int, masked_fill_zero: bool, weight_from_c: bool,
+                   renorm: bool, scale: float, eps: float, want_logits: bool = False, round_logits_bf16: bool = False):
+    """Gate projection and router in one library call: ``self.gate.forward(hidden_states.float())`` +
+    ``FusedMoE.select_experts`` (deepseek_moe.py:147-152,253-256).  ``x`` [T,H] bf16 or fp32 is read as it
+    is (no fp32 copy), ``gate_w`` [E,H] fp32 or bf16.  ``top_k`` = 0 computes the logits only.
+    Returns (topk_w, topk_ids, logits or None)."""
+    _need_gpu(x, gate_w, bias)
+    if x.dim() != 2 or gate_w.dim() != 2 or x.shape[1] != gate_w.shape[1]:
+        raise ValueError("gate: x must be [T, H] and the gate weight [E, H]")
+    if x.dtype not in (torch.bfloat16, torch.float32) or gate_w.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("gate: tokens and gate weight must be bf16 or fp32")
+    x = x.contiguous()
+    gate_w = gate_w.contiguous()
+    T, H = x.shape
+    E = gate_w.shape[0]
+    dev = x.device
+    if bias is not None:
+        bias = bias.float().contiguous()
+        if bias.numel() != E:
+            raise ValueError("bias must have one entry per expert")
+    fn = {"softmax": L.OMNI_SCORE_SOFTMAX, "sigmoid": L.OMNI_SCORE_SIGMOID}.get(score_fn)
+    if fn is None:
+        raise ValueError(f"Unsupported scoring function: {score_fn}")
+    need = L.lib().omni_moe_gate_route_workspace_bytes(T, H, E)
+    key = str(dev)
+    ws = _GATE_WS.get(key)   # one scratch per device, grown on demand; calls on one stream are ordered
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        _GATE_WS[key] = ws
+    w = torch.empty(T, top_k, dtype=torch.float32, device=dev) if top_k > 0 else None
+    ids = torch.empty(T, top_k, dtype=torch.int32, device=dev) if top_k > 0 else None
+    logits = torch.empty(T, E, dtype=torch.float32, device=dev) if (want_logits or top_k == 0) else None
+    rc = L.lib().omni_moe_gate_route(_ptr(x), _DT[x.dtype], _ptr(gate_w), _DT[gate_w.dtype], _ptr(bias), T, H, E,
+                                     int(n_group), int(topk_group), int(top_k), fn, int(group_mode),
+                                     int(masked_fill_zero), int(weight_from_c), int(renorm), float(scale), float(eps),
+                                     int(round_logits_bf16), _ptr(logits), _ptr(w), _ptr(ids), _ptr(ws), ws.numel(),
+                                     _stream())
+    L.check(rc, "omni_moe_gate_route")
+    return w, ids, logits
+
+
+def gate_logits(x: torch.Tensor, gate_w: torch.Tensor, round_logits_bf16: bool = False) -> torch.Tensor:
+    """``ReplicatedLinear.forward`` of the gate (deepseek_moe.py:147-152): fp32 logits [T, E] in the
+    library's fixed summation order."""
+    return moe_gate_route(x, gate_w, None, 0, 1, 1, "softmax", L.OMNI_GROUP_MAX, False, False, False, 1.0, 0.0,
+                          round_logits_bf16=round_logits_bf16)[2]
+
+
+_ROW_IDX = {}
+
+
 def _row_idx(T: int, K: int, device) -> torch.Tensor:
-    # row_idx[n, k] = k*T + n (fused_moe.py:80-81, layer.py:352-353)
-    return torch.arange(T * K, device=device, dtype=torch.int32).view(K, T).transpose(0, 1)
+    """row_idx[n, k] = k*T + n (fused_moe.py:80-81, layer.py:352-353).  A constant of (T, K): made once per
+    shape and device, so that the routing wrappers launch nothing but the router."""
+    key = (int(T), int(K), str(device))
+    t = _ROW_IDX.get(key)
+    if t is None:
+        if len(_ROW_IDX) > 256:
+            _ROW_IDX.clear()
+        t = torch.arange(T * K, device=device, dtype=torch.int32).view(K, T).transpose(0, 1)
+        _ROW_IDX[key] = t
+    return t
 
 
 def npu_moe_gating_top_k(x: torch.Tensor, k: int, bias: Optional[torch.Tensor], k_group: int, group_count: int,

@@ -124,12 +124,21 @@ class DeepseekMoE(nn.Module):
                     lin.quant_method.process_weights_after_loading(lin)
 
     def _route(self, hidden_states):
-        router_logits, _ = self.gate.forward(hidden_states.float())
+        """``self.gate.forward(hidden_states.float())`` + ``FusedMoE.select_experts`` (deepseek_moe.py:253-256,
+        329-333).  The fused body makes both in one library call on the tokens as they are; the
+        operator-by-operator body keeps the reference's two steps.  Same bits either way."""
         e = self.experts
-        topk_weights, topk_ids, _ = FusedMoE.select_experts(
-            hidden_states, router_logits, e.top_k, e.use_grouped_topk, e.renormalize, e.topk_group,
-            e.num_expert_group, e.custom_routing_function, e.scoring_func, e.e_score_correction_bias,
-            self.routed_scaling_factor, layer=e)
+        if self.fused:
+            topk_weights, topk_ids, _, _ = FusedMoE.gate_and_select_experts(
+                hidden_states, self.gate.weight, e.top_k, e.use_grouped_topk, e.renormalize, e.topk_group,
+                e.num_expert_group, e.custom_routing_function, e.scoring_func, e.e_score_correction_bias,
+                self.routed_scaling_factor)
+        else:
+            router_logits, _ = self.gate.forward(hidden_states.float())
+            topk_weights, topk_ids, _ = FusedMoE.select_experts(
+                hidden_states, router_logits, e.top_k, e.use_grouped_topk, e.renormalize, e.topk_group,
+                e.num_expert_group, e.custom_routing_function, e.scoring_func, e.e_score_correction_bias,
+                self.routed_scaling_factor, layer=e)
         return topk_weights, e.apply_expert_load_balance(topk_ids=topk_ids)
 
     def forward(self, hidden_states: torch.Tensor, residual: torch.Tensor, attn_metadata, layer_id: int = 0,

@@ -108,6 +108,51 @@ class FusedMoE(torch.nn.Module):
                 hidden_states=hidden_states, gating_output=router_logits, topk=top_k, renormalize=renormalize)
         return topk_weights, topk_ids, row_idx
 
+    @staticmethod
+    def gate_and_select_experts(hidden_states: torch.Tensor, gate_weight: torch.Tensor, top_k: int,
+                                use_grouped_topk: bool, renormalize: bool, topk_group: Optional[int] = None,
+                                num_expert_group: Optional[int] = None,
+                                custom_routing_function: Optional[Callable] = None, scoring_func: str = "softmax",
+                                e_score_correction_bias: Optional[torch.Tensor] = None,
+                                routed_scaling_factor: Optional[float] = None, want_logits: bool = False):
+        """``gate.forward(hidden_states.float())`` followed by ``select_experts`` (deepseek_moe.py:253-256,
+        329-333) as one library call: the tokens are read as they are (no fp32 copy), the logits are summed
+        in the library's fixed order and routed by the same three routers with the same arguments as
+        ``select_experts`` gives them.  Returns (topk_weights, topk_ids, row_idx, router_logits or None)."""
+        L = ops.L
+        bf16_gate = gate_weight.dtype == torch.bfloat16
+        T = hidden_states.shape[0]
+        if use_grouped_topk:
+            if topk_group is None:
+                raise ValueError("Unsupported topk_group is None")
+            if num_expert_group is None:
+                raise ValueError("Unsupported num_expert_group is None")
+            if e_score_correction_bias is None:
+                if scoring_func not in ("softmax", "sigmoid"):
+                    raise ValueError(f"Unsupported scoring function: {scoring_func}")
+                # grouped_topk (fused_moe.py:38-84), then the scaling factor (layer.py:339)
+                w, ids, logits = ops.moe_gate_route(hidden_states, gate_weight, None, top_k, num_expert_group, topk_group,
+                                                    scoring_func, L.OMNI_GROUP_MAX, True, True, bool(renormalize), 1.0,
+                                                    0.0, want_logits, bf16_gate)
+                w = w * routed_scaling_factor
+            else:
+                # npu_moe_gating_top_k as called at layer.py:341-351
+                w, ids, logits = ops.moe_gate_route(hidden_states, gate_weight, e_score_correction_bias, top_k,
+                                                    num_expert_group, topk_group, "sigmoid", L.OMNI_GROUP_TOP2SUM, False,
+                                                    False, True, routed_scaling_factor, float(1e-20), want_logits,
+                                                    bf16_gate)
+        elif custom_routing_function is None:
+            # fused_topk (fused_moe.py:24-34)
+            w, ids, logits = ops.moe_gate_route(hidden_states, gate_weight, None, top_k, 1, 1, "softmax",
+                                                L.OMNI_GROUP_MAX, False, False, bool(renormalize), 1.0, 0.0, want_logits,
+                                                bf16_gate)
+        else:
+            logits = ops.gate_logits(hidden_states, gate_weight, round_logits_bf16=bf16_gate)
+            w, ids, row_idx = custom_routing_function(hidden_states=hidden_states, gating_output=logits, topk=top_k,
+                                                      renormalize=renormalize)
+            return w, ids, row_idx, logits
+        return w, ids, ops._row_idx(T, top_k, hidden_states.device), logits
+
     def forward(self, hidden_states: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
                 pertoken_scale: torch.Tensor, attn_metadata, comm_group=None):
         """layer.py:384-408 (the all-reduce of a tensor-parallel expert split is not built:

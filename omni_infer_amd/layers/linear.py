@@ -30,7 +30,16 @@ class ReplicatedLinear(nn.Module):
 
     def forward(self, x):
         if self.quant_method is None:
-            return torch.nn.functional.linear(x, self.weight), None
+            # the unquantised replicated linear of the MoE path is the gate (deepseek_moe.py:147-152): its
+            # product runs on the fp32 matrix cores in the library's fixed summation order; a bf16 gate
+            # (deepseek_v3_a2.py:607-613) hands back bf16 logits
+            from .. import hip_ops as ops
+            lead = x.shape[:-1]
+            bf16_gate = self.weight.dtype == torch.bfloat16
+            logits = ops.gate_logits(x.reshape(-1, x.shape[-1]), self.weight, round_logits_bf16=bf16_gate)
+            if bf16_gate:
+                logits = logits.to(torch.bfloat16)
+            return logits.view(*lead, self.output_size), None
         return self.quant_method.apply_weights(self, x, None), None
 
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor) -> None:

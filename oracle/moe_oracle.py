@@ -31,6 +31,10 @@ tests/test_oracle_pins.py):
 
 * exp_spec / sigmoid_spec / silu_spec ... torch.exp / sigmoid / F.silu within
   4 ulp over a dense sweep; monotonicity; exact values at 0.
+* fma32 / gate_logits_spec ... exact rational arithmetic (fractions) on random
+  and constructed half-way cases; fp64 matmul (a dropped term, a transposed
+  operand or a wrong slice boundary fails); invariance under the split of the
+  slices over wavefronts is a property of the device test.
 * route_noaux_tc ........ transformers DeepseekV3TopkRouter arithmetic
   (library routine, ids as sets + weights), brute force over all subsets on
   tiny E, invariants (distinct ids, group membership, sum of weights).
@@ -125,6 +129,68 @@ def silu_spec(x: torch.Tensor) -> torch.Tensor:
     """x / (1 + exp_spec(-x))."""
     x = x.to(F32)
     return x / (_c(1.0) + exp_spec(-x))
+
+
+# --------------------------------------------------------------------------
+# Gate projection with a stated summation order
+# --------------------------------------------------------------------------
+GATE_SLICE = 128   # reduction elements of one fused-multiply-add chain
+GATE_GROUP = 8     # slices added up before the groups are
+
+
+def fma32(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> torch.Tensor:
+    """fp32 fused multiply-add, a*b + c with a single rounding (round to nearest even), for fp32
+    tensors without overflow or subnormal results.
+
+    The product of two fp32 numbers is exact in fp64 (48 significant bits).  The fp64 sum p + c is
+    rounded once to 53 bits; rounding that again to 24 bits differs from the single rounding only when
+    the fp64 sum lies exactly half way between two neighbouring fp32 numbers while the exact sum does
+    not.  The exact error of the fp64 addition (two-sum) tells on which side the exact sum lies."""
+    p = a.to(torch.float64) * b.to(torch.float64)
+    cd = c.to(torch.float64)
+    s = p + cd
+    r = s.to(F32)
+    bb = s - p
+    err = (p - (s - bb)) + (cd - bb)                       # exact: s + err == p + c
+    rd = r.to(torch.float64)
+    toward = torch.where(s > rd, torch.full_like(r, float("inf")), torch.full_like(r, float("-inf")))
+    other = torch.nextafter(r, toward)
+    tie = (rd != s) & ((rd - s).abs() == (other.to(torch.float64) - s).abs())
+    fix = tie & (err != 0)
+    if bool(fix.any()):
+        hi = torch.maximum(r, other)
+        lo = torch.minimum(r, other)
+        r = torch.where(fix, torch.where(err > 0, hi, lo), r)
+    return r
+
+
+def gate_logits_spec(x: torch.Tensor, w: torch.Tensor, round_bf16: bool = False) -> torch.Tensor:
+    """``router_logits, _ = self.gate.forward(hidden_states.float())`` (omni/models/common/layers/moe/
+    deepseek_moe.py:147-152,253,329): logits[t,e] = sum_k x[t,k] * w[e,k] in fp32, here with the stated
+    order of the device library (the reference leaves the order to its BLAS):
+
+    the reduction is cut into slices of 128 elements; a slice is a chain of fused multiply-adds over
+    ascending k starting from +0; 8 consecutive slices are added left to right into a group sum; the
+    group sums are added left to right.  ``round_bf16``: the bf16 gate of deepseek_v3_a2.py:607-613
+    hands bf16 logits to the router.  x [T,H] (bf16 or fp32), w [E,H] (fp32 or bf16), H % 128 == 0."""
+    xf, wf = x.to(F32), w.to(F32)
+    T, H = xf.shape
+    E = wf.shape[0]
+    assert H % GATE_SLICE == 0
+    n_slices = H // GATE_SLICE
+    wt = wf.t().contiguous()                                # [H, E]
+    total = None
+    for g0 in range(0, n_slices, GATE_GROUP):
+        q = None
+        for s_ in range(g0, min(g0 + GATE_GROUP, n_slices)):
+            acc = torch.zeros(T, E, dtype=F32)
+            for k in range(s_ * GATE_SLICE, (s_ + 1) * GATE_SLICE):
+                acc = fma32(xf[:, k:k + 1], wt[k:k + 1, :], acc)
+            q = acc if q is None else q + acc
+        total = q if total is None else total + q
+    if round_bf16:
+        total = total.to(torch.bfloat16).to(F32)
+    return total
 
 
 # --------------------------------------------------------------------------

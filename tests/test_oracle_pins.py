@@ -477,3 +477,86 @@ def test_deepseek_moe_forward_against_fp64_witness():
     assert torch.equal(out, out_wo + sh)
     fp32_add = (st["out32"] + _fp64_shared(x, *lay.shared).float()).to(torch.bfloat16)
     assert not torch.equal(out, fp32_add)                          # and that is a different number
+
+
+# ------------------------------------------------------------------ gate projection with a stated order
+def _fma_exact(a: float, b: float, c: float) -> float:
+    """a*b + c in exact rational arithmetic, rounded once to fp32 (round to nearest even)."""
+    from fractions import Fraction
+    v = Fraction(a) * Fraction(b) + Fraction(c)
+    if v == 0:
+        return 0.0
+    f = np.float32(float(v))                     # a first guess; fix it with exact comparisons
+    cands = sorted({float(np.nextafter(f, np.float32(-np.inf))), float(f), float(np.nextafter(f, np.float32(np.inf)))})
+    best = min(cands, key=lambda t: (abs(Fraction(t) - v), int(np.float32(t).view(np.uint32)) & 1))
+    return best
+
+
+def test_fma32_is_a_single_rounding():
+    g = gen(40)
+    a = torch.randn(4000, generator=g) * 3
+    b = torch.randn(4000, generator=g) * 0.05
+    c = torch.randn(4000, generator=g) * torch.logspace(-6, 6, 4000)
+    # constructed double-rounding traps: c has an odd last mantissa bit, a*b is half an ulp of c minus (or
+    # plus) something far below the fp64 resolution at c, so the fp64 sum is exactly the half-way point and a
+    # second rounding would go to the even neighbour whatever side the exact sum is on
+    traps_a, traps_b, traps_c = [], [], []
+    eps = 2.0 ** -23
+    for e in (10, 20, 30):
+        for sa, sb in ((1, -1), (1, 1), (-1, -1)):
+            for csign in (1.0, -1.0):
+                c_val = csign * (2.0 ** e) * (1 + eps)                 # odd mantissa
+                half_ulp = 2.0 ** (e - 24)
+                root = 2.0 ** ((e - 24) / 2) if (e - 24) % 2 == 0 else None
+                if root is None:
+                    continue
+                traps_a.append(csign * root * (1 + sa * eps))
+                traps_b.append(root * (1 + sb * eps))                  # a*b = +-half_ulp * (1 +- 2^-22.. or -2^-46)
+                traps_c.append(c_val)
+    a = torch.cat([a, torch.tensor(traps_a)]).float()
+    b = torch.cat([b, torch.tensor(traps_b)]).float()
+    c = torch.cat([c, torch.tensor(traps_c)]).float()
+    got = O.fma32(a, b, c)
+    want = torch.tensor([_fma_exact(float(x), float(y), float(z)) for x, y, z in zip(a, b, c)], dtype=torch.float32)
+    assert torch.equal(got, want)
+    naive = (a.double() * b.double() + c.double()).float()
+    assert not torch.equal(naive, want), "the traps do not trap: fp64 then fp32 rounding agreed everywhere"
+    two_roundings = a * b + c
+    assert not torch.equal(two_roundings, want)
+
+
+def test_gate_logits_spec_against_fp64_matmul():
+    g = gen(41)
+    T, H, E = 9, 1024, 40
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w = torch.randn(E, H, generator=g) * 0.02
+    got = O.gate_logits_spec(x, w)
+    ref = x.double() @ w.double().t()
+    assert got.shape == (T, E) and got.dtype == torch.float32
+    assert float((got.double() - ref).abs().max()) < 2e-6 * float(ref.abs().max()) + 1e-6
+    # mistakes this must catch: a transposed operand, a dropped slice, a dropped last element
+    assert rel_err(got, x.double() @ w.double().flip(1).t()) > 0.5
+    assert float((got.double() - x.double()[:, 128:] @ w.double()[:, 128:].t()).abs().max()) > 1e-3
+    assert float((got.double() - x.double()[:, :-1] @ w.double()[:, :-1].t()).abs().max()) > 1e-5
+    # the order is the stated one: chains of 128, groups of 8 slices.  A plain left-to-right fp32 sum differs
+    # in the last bits, the stated tree reproduced with python floats (exact fma per step) does not
+    t, e = 3, 17
+    xs, ws = x[t].float().tolist(), w[e].tolist()
+    slices = []
+    for s0 in range(0, H, 128):
+        acc = 0.0
+        for k in range(s0, s0 + 128):
+            acc = _fma_exact(xs[k], ws[k], acc)
+        slices.append(np.float32(acc))
+    tot = None
+    for g0 in range(0, len(slices), 8):
+        q = slices[g0]
+        for v in slices[g0 + 1:g0 + 8]:
+            q = np.float32(q + v)
+        tot = q if tot is None else np.float32(tot + q)
+    assert float(got[t, e]) == float(tot)
+    # bf16 weights and the bf16-rounded output of the bf16 gate
+    wb = w.to(torch.bfloat16)
+    got_b = O.gate_logits_spec(x, wb, round_bf16=True)
+    assert torch.equal(got_b, got_b.to(torch.bfloat16).float())
+    assert float((got_b.double() - x.double() @ wb.double().t()).abs().max()) < 0.01 * float(ref.abs().max())
