@@ -385,14 +385,66 @@ def measure_block(name, ws, steps, warmup, dev):
             "tokens": T}
 
 
+def bench_calib(args):
+    """What the hardware delivers on this box, to read the layer's figures against (one JSON line):
+    the int8 matrix instruction alone on zero and on random operands, the vendor library's plain int8 GEMM
+    (torch._int_mm) at the shapes of the two prefill GEMMs, and a device-to-device copy."""
+    from omni_infer_amd import _lib as L
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib, st = L.lib(), torch.cuda.current_stream().cuda_stream
+    props = torch.cuda.get_device_properties(dev)
+    cus = props.multi_processor_count
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    res = {"metric": "hardware_calibration", "unit": "POPS", "n_gpus": 1, "data": "synthetic", "cus": cus,
+           "int8_peak_published_pops": INT8_PEAK / 1e15}
+
+    def ev_ms(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    iters, g = 20000, torch.Generator(device=dev).manual_seed(0)
+    for name, ops_buf in (("zeros", torch.zeros(1 << 16, dtype=torch.int8, device=dev)),
+                          ("random_uniform", torch.randint(-128, 128, (1 << 16,), generator=g, device=dev, dtype=torch.int8)),
+                          ("gaussian_sigma30", (torch.randn(1 << 16, generator=g, device=dev) * 30).clamp(-127, 127).to(torch.int8))):
+        def run():
+            L.check(lib.omni_diag_mfma_i8_rate(ops_buf.data_ptr(), ops_buf.numel(), iters, cus, sink.data_ptr(), st),
+                    "omni_diag_mfma_i8_rate")
+        ms = ev_ms(run, 5)
+        ops_total = cus * 8 * 8 * iters * 65536.0
+        res[f"mfma_i8_{name}_pops"] = ops_total / (ms * 1e-3) / 1e15
+        res[f"mfma_i8_{name}_ms"] = ms
+    for tag, (M, K, N) in (("gemm1_shape", (65536, 7168, 4096)), ("gemm2_shape", (65536, 2048, 7168))):
+        a = torch.randint(-128, 128, (M, K), generator=g, device=dev, dtype=torch.int8)
+        b = torch.randint(-128, 128, (N, K), generator=g, device=dev, dtype=torch.int8).t()   # column-major B
+        ms = ev_ms(lambda: torch._int_mm(a, b), 5)
+        res[f"vendor_int_mm_{tag}_pops"] = 2.0 * M * K * N / (ms * 1e-3) / 1e15
+        res[f"vendor_int_mm_{tag}_us"] = ms * 1e3
+        del a, b
+    src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    ms = ev_ms(lambda: dst.copy_(src), 10)
+    res["copy_1GiB_read_plus_write_TBps"] = 2 * (1 << 30) / (ms * 1e-3) / 1e12
+    res["value"] = res["mfma_i8_gaussian_sigma30_pops"]
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=4000, help="timed decode steps (prefill runs steps/100, at least 10)")
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", choices=["all", "decode", "prefill", "norm"], default="all",
+    ap.add_argument("--workload", choices=["all", "decode", "prefill", "norm", "calib"], default="all",
                     help="all (default): decode headline + prefill object + block_us; decode / prefill: that half only; "
-                         "norm: the RMSNorm+quant producer")
+                         "norm: the RMSNorm+quant producer; calib: what the hardware delivers (matrix instruction "
+                         "alone, vendor int8 GEMM, copy)")
     ap.add_argument("--rows", choices=["f32", "bf16"], default="f32",
                     help="row dtype between GEMM2 and the combine (the product default is f32)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -409,6 +461,8 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "calib":
+        return bench_calib(args)
     if args.workload == "norm":
         if args.steps == 4000:
             args.steps, args.warmup = 200, 20

@@ -220,6 +220,15 @@ int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int
                               size_t buf_bytes);
 
 /*
+ * Diagnostic (no counterpart in the reference): the sustained rate of v_mfma_i32_32x32x32_i8 on given operand
+ * bits with nothing else in the loop.  `blocks` blocks of 8 wavefronts each issue 8 * iters instructions per
+ * wavefront (65 536 op each) on operands taken from `operands` (>= 64 KiB; zeros and random bits give different
+ * rates because the chip lowers its clock with the switching activity).  The caller times the launch.
+ */
+int omni_diag_mfma_i8_rate(const int8_t* operands, size_t operand_bytes, int iters, int blocks, int32_t* sink,
+                           void* stream);
+
+/*
  * Weighted un-permute.  Replaces the routing half of npu_grouped_matmul_finalize_routing
  * (fused_moe.py:536), npu_moe_finalize_routing (compressed_tensors_moe.py:253;
  * deepseek_moe.py:292-301) and the shared-expert add (deepseek_moe.py:303,366).
