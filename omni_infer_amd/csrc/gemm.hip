@@ -626,8 +626,9 @@ struct Plan {
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
+//   OMNI_MOE_EQUAL_PROGRESS 0: the stream kernel of GEMM1 leaves the issue priority of its wavefronts alone
 struct Tuning {
-  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0;
+  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1;
   bool have[3] = {false, false, false};
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
@@ -644,6 +645,7 @@ const Tuning& tuning() {
     r.tile_tail = geti("OMNI_MOE_TILE_TAIL", 1);
     r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
     r.rowq = geti("OMNI_MOE_ROWQ", 0);
+    r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
     for (int kind = 1; kind <= 2; ++kind) {
       const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
       const char* e = getenv(name);
@@ -731,10 +733,14 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
 }
 
 template <int KIND, int MT, int NT, int D>
-void launch_stream(const GemmArgs& a, int64_t M_cap, int units, hipStream_t st) {
+void launch_stream(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
+  GemmArgs a = a0;
   const int BM = 16 * MT;
   const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
   int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
+  // GEMM1 (every block resident at once, long streams) gains from equal progress; GEMM2 (three rounds of short
+  // blocks, where the older round should finish first and make room) loses by it: measured 84.4 -> 87.6 us
+  a.equal_progress = (KIND == 1 && a.S == 1) ? tuning().equal_progress : 0;
   dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks, (unsigned)a.S), block(256);
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }

@@ -31,6 +31,7 @@ struct GemmArgs {
   int32_t* tail_part;             // tile kernel: partial accumulators of the split tiles
   int32_t* part;       // GEMM1 stream kernel: [S, M_cap, N] partial accumulators (split-k)
   int S;               // number of k splits (grid.z)
+  int equal_progress;  // stream kernel: a wavefront lowers its issue priority as it advances through k
   int64_t M_cap;
 };
 
@@ -88,7 +89,7 @@ constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1
 // (block barriers inside); when it returns nobody reads the LDS buffers any more.
 template <int KIND, int MT, int NT, int D, typename BeforeA>
 __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& rb, int bx, int bz,
-                                             v4i (*lds_a)[MT * 4 * WAVE], BeforeA before_a) {
+                                             v4i (*lds_a)[MT * 4 * WAVE], float* lds_ts, BeforeA before_a) {
   constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
   constexpr int DC = D / 4;                       // chunks (4 k-steps) of B in flight
   static_assert(D % 4 == 0, "D counts whole chunks");
@@ -131,6 +132,10 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
     for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
   __builtin_amdgcn_sched_barrier(0);
   before_a();
+  // the activation scale of every row of the block goes to LDS now (one or two dependent loads per row, whose
+  // way is then covered by the k loop instead of standing in front of the epilogue)
+  if (threadIdx.x < 16 * MT)
+    lds_ts[threadIdx.x] = ((int)threadIdx.x < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + threadIdx.x)] : 0.0f;
 
   // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile, k-step w of
   // every chunk; rows past the end of the group alias the group's first row
@@ -189,7 +194,20 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
   };
 
   int c0 = 0;
+  // Wavefronts of one SIMD are served oldest first, so without help the blocks of a launch that is resident
+  // all at once finish in the order they started and the last ones stream alone, with too few loads in
+  // flight to fill the memory system.  With a.equal_progress a wavefront lowers its issue priority by one level
+  // per quarter of its reduction: wavefronts that are behind overtake those ahead, all of them finish
+  // together, and the thin tail is gone (GEMM1 of the decode call: 162.7 -> 159.1 us).
+  const bool equal_progress = a.equal_progress;
   for (; c0 < nchunks - DC; c0 += DC) {
+    if (equal_progress) {
+      const int q = (c0 * 4) / nchunks;
+      if (q == 0) __builtin_amdgcn_s_setprio(3);
+      else if (q == 1) __builtin_amdgcn_s_setprio(2);
+      else if (q == 2) __builtin_amdgcn_s_setprio(1);
+      else __builtin_amdgcn_s_setprio(0);
+    }
 #pragma unroll
     for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, true);
   }
@@ -209,8 +227,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
           const int rbase = mt * 16 + 4 * (lane >> 4);
           float ts[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            ts[i] = (rbase + i < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rbase + i)] : 0.0f;
+          for (int i = 0; i < 4; ++i) ts[i] = lds_ts[rbase + i];
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
             const int n = strip[2 * t] * 16 + col;
@@ -253,10 +270,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
         const int rbase = mt * 16 + 4 * (lane >> 4);
         float ts[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          int rr = rbase + i;
-          ts[i] = (rr < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + rr)] : 0.0f;
-        }
+        for (int i = 0; i < 4; ++i) ts[i] = lds_ts[rbase + i];
 #pragma unroll
         for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsc, strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
       }
@@ -267,9 +281,10 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 template <int KIND, int MT, int NT, int D>
 __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void gemm_stream(GemmArgs a) {
   __shared__ v4i lds_a[2][MT * 4 * WAVE];
+  __shared__ float lds_ts[16 * MT];
   RowBlock rb;
   if (!find_row_block(a.offsets, a.G, a.extra_rows, 16 * MT, blockIdx.y, rb)) return;
-  stream_block<KIND, MT, NT, D>(a, rb, blockIdx.x, blockIdx.z, lds_a, [] {});
+  stream_block<KIND, MT, NT, D>(a, rb, blockIdx.x, blockIdx.z, lds_a, lds_ts, [] {});
 }
 
 // Row quantisation of y = silu(gate) * up (fp32) by one wavefront: scale = max|y| / 127, q = rint(y / scale).
