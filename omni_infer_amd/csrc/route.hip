@@ -19,6 +19,7 @@
 //       logits = Q_0 + Q_1 + ... (left to right).
 //   How the slices are dealt to wavefronts (one slice each for small batches, one group each for
 //   large ones) does not change a bit of the result.
+#include <stdlib.h>
 #include "common.h"
 
 namespace {
@@ -369,11 +370,171 @@ __global__ __launch_bounds__(64) void gate_partial_kernel(GateArgs a) {
   }
 }
 
+// ---------------------------------------------------------------- gate projection, large batches
+// Block of four wavefronts: 128 tokens x 64 experts x one group of 8 slices, a wavefront 64 x 32 as above.
+// The operands pass through LDS: every 16-byte global load covers consecutive bytes of one row (the one-
+// wavefront kernel asks for 64 different cache lines per load instruction, which is what limits it once the
+// batch is large), each wavefront then reads "its" row per lane (token 64 (w&1) + l, expert 32 (w>>1) + l%32)
+// with 16-byte LDS reads; rows are padded by 16 bytes, so the 16 lanes that LDS serves together hit 16
+// different groups of four banks.  Stages of 32 reduction elements, two LDS buffers, the global loads of the
+// next stage are in flight while the current one is multiplied; one barrier per stage; three blocks per CU.
+// The order of the multiply-adds and of the sums is that of the one-wavefront kernel: the same bits.
+// (Two chains per wavefront against the same tokens, alternating so that no matrix instruction directly
+// follows the one it accumulates onto, was measured and is not faster.)
+constexpr int GT_TOK = 128, GT_EXP = 64, GT_KS = 32;
+
+template <int DT>
+struct LdsChunk16;  // 16 consecutive reduction elements of one LDS row
+template <>
+struct LdsChunk16<OMNI_DT_F32> {
+  v4f r[4];
+  __device__ __forceinline__ void load(const unsigned char* row, int k) {
+    const v4f* p = (const v4f*)(row + k * 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = p[i];
+  }
+  __device__ __forceinline__ float at(int k) const { return r[k >> 2][k & 3]; }
+};
+template <>
+struct LdsChunk16<OMNI_DT_BF16> {
+  v4i r[2];
+  __device__ __forceinline__ void load(const unsigned char* row, int k) {
+    const v4i* p = (const v4i*)(row + k * 2);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) r[i] = p[i];
+  }
+  __device__ __forceinline__ float at(int k) const {
+    const uint32_t word = (uint32_t)r[k >> 3][(k >> 1) & 3];
+    return __uint_as_float((k & 1) ? (word & 0xffff0000u) : (word << 16));
+  }
+};
+
+template <int XDT, int WDT>
+__global__ __launch_bounds__(256, (XDT == OMNI_DT_F32 && WDT == OMNI_DT_F32) ? 2 : 3) void gate_tile_kernel(GateArgs a) {
+  constexpr int XES = (XDT == OMNI_DT_F32) ? 4 : 2, WES = (WDT == OMNI_DT_F32) ? 4 : 2;
+  constexpr int XROW = GT_KS * XES + 16, WROW = GT_KS * WES + 16;  // bytes of a padded LDS row
+  constexpr int XBUF = GT_TOK * XROW, WBUF = GT_EXP * WROW;
+  constexpr int XCPR = GT_KS * XES / 16, WCPR = GT_KS * WES / 16;  // 16-byte pieces of a row's stage
+  constexpr int XN = GT_TOK * XCPR / 256, WN = GT_EXP * WCPR / 256;  // pieces per thread
+  constexpr int SPS = GATE_SLICE / GT_KS;                           // stages per slice
+  static_assert(XN >= 1 && WN >= 1 && GT_KS % 16 == 0, "stage too small for 256 threads");
+  __shared__ __align__(16) unsigned char lds[2 * (XBUF + WBUF)];
+
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
+  int id = blockIdx.x;
+  const int tt = id % a.n_tt; id /= a.n_tt;
+  const int et = id % a.n_et; id /= a.n_et;
+  const int part = id;
+  const int n_slices = a.H / GATE_SLICE;
+  const int s_first = part * GATE_GROUP;
+  const int s_end = min(n_slices, s_first + GATE_GROUP);
+  const int n_st = (s_end - s_first) * SPS;
+  const size_t k_first = (size_t)s_first * GATE_SLICE;
+
+  // what this thread carries from global memory to LDS (rows past the end alias the last row; not stored)
+  const char* xsrc[XN];
+  const char* wsrc[WN];
+  int xdst[XN], wdst[WN];
+#pragma unroll
+  for (int i = 0; i < XN; ++i) {
+    const int c = i * 256 + tid, row = c / XCPR, col = c % XCPR;
+    xsrc[i] = (const char*)a.x + ((size_t)min(tt * GT_TOK + row, a.T - 1) * a.H + k_first) * XES + col * 16;
+    xdst[i] = row * XROW + col * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < WN; ++i) {
+    const int c = i * 256 + tid, row = c / WCPR, col = c % WCPR;
+    wsrc[i] = (const char*)a.w + ((size_t)min(et * GT_EXP + row, a.E - 1) * a.H + k_first) * WES + col * 16;
+    wdst[i] = XBUF + row * WROW + col * 16;
+  }
+  v4i xg[XN], wg[WN];
+#pragma unroll
+  for (int i = 0; i < XN; ++i) xg[i] = *(const v4i*)xsrc[i];
+#pragma unroll
+  for (int i = 0; i < WN; ++i) wg[i] = *(const v4i*)wsrc[i];
+#pragma unroll
+  for (int i = 0; i < XN; ++i) *(v4i*)(lds + xdst[i]) = xg[i];
+#pragma unroll
+  for (int i = 0; i < WN; ++i) *(v4i*)(lds + wdst[i]) = wg[i];
+  __syncthreads();
+
+  const int xrow_off = ((wv & 1) * 64 + lane) * XROW;
+  const int wrow_off = XBUF + ((wv >> 1) * 32 + (lane & 31)) * WROW;
+  v32f acc, q;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) { acc[i] = 0.0f; q[i] = 0.0f; }
+  for (int st = 0; st < n_st; ++st) {
+    const int st_next = min(st + 1, n_st - 1);  // the last stage is requested once more instead of a branch
+#pragma unroll
+    for (int i = 0; i < XN; ++i) xg[i] = *(const v4i*)(xsrc[i] + (size_t)st_next * GT_KS * XES);
+#pragma unroll
+    for (int i = 0; i < WN; ++i) wg[i] = *(const v4i*)(wsrc[i] + (size_t)st_next * GT_KS * WES);
+    const unsigned char* buf = lds + (st & 1) * (XBUF + WBUF);
+    LdsChunk16<XDT> xc[2];
+    LdsChunk16<WDT> wc[2];
+    xc[0].load(buf + xrow_off, 0);
+    wc[0].load(buf + wrow_off, 0);
+    // the scheduling barriers keep the requests where they are written: the global loads a whole stage, the
+    // LDS reads sixteen steps ahead of their use
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < GT_KS / 16; ++j) {
+      if (j + 1 < GT_KS / 16) {
+        xc[(j + 1) & 1].load(buf + xrow_off, (j + 1) * 16);
+        wc[(j + 1) & 1].load(buf + wrow_off, (j + 1) * 16);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int k = 0; k < 16; ++k)
+        acc = __builtin_amdgcn_mfma_f32_32x32x1f32(xc[j & 1].at(k), wc[j & 1].at(k), acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    unsigned char* nbuf = lds + ((st + 1) & 1) * (XBUF + WBUF);
+#pragma unroll
+    for (int i = 0; i < XN; ++i) *(v4i*)(nbuf + xdst[i]) = xg[i];
+#pragma unroll
+    for (int i = 0; i < WN; ++i) *(v4i*)(nbuf + wdst[i]) = wg[i];
+    __syncthreads();
+    if ((st & (SPS - 1)) == SPS - 1) {
+      // the slice's chain is complete: add it to the group's sum (the first slice starts it)
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        q[i] = (st < SPS) ? acc[i] : q[i] + acc[i];
+        acc[i] = 0.0f;
+      }
+    }
+  }
+  float* out = a.partials + (size_t)part * a.T * a.E;
+  const int e = et * GT_EXP + (wv >> 1) * 32 + (lane & 31);
+  if (e < a.E) {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const int t = tt * GT_TOK + (wv & 1) * 64 + 32 * (i >> 4) + 8 * ((i & 15) >> 2) + 4 * (lane >> 5) + (i & 3);
+      if (t < a.T) out[(size_t)t * a.E + e] = q[i];
+    }
+  }
+}
+
+// Tuning aids, read from the environment once.
+struct GateTuning {
+  int group_tasks;  // from this many (64 tokens x 32 experts x group) tasks on, a task is a whole group of slices
+  int tile_from;    // from this many tokens on, the block kernel that passes the operands through LDS
+};
+const GateTuning& gate_tuning() {
+  static const GateTuning t = [] {
+    GateTuning g{400, 1024};
+    if (const char* e = getenv("OMNI_MOE_GATE_GROUP_TASKS")) { const int v = atoi(e); if (v > 0) g.group_tasks = v; }
+    if (const char* e = getenv("OMNI_MOE_GATE_TILE_FROM")) { const int v = atoi(e); if (v > 0) g.tile_from = v; }
+    return g;
+  }();
+  return t;
+}
+
 // small batches: one slice per wavefront (many short tasks); large ones: a group of 8 slices each
 int gate_slices_per_task(int T, int H, int E) {
   const int n_tt = (T + 63) / 64, n_et = (E + 31) / 32;
   const int n_groups = (H / GATE_SLICE + GATE_GROUP - 1) / GATE_GROUP;
-  return ((int64_t)n_tt * n_et * n_groups >= 1024) ? GATE_GROUP : 1;
+  return ((int64_t)n_tt * n_et * n_groups >= gate_tuning().group_tasks) ? GATE_GROUP : 1;
 }
 
 void launch_route(const RouteArgs& a, hipStream_t st) {
@@ -449,16 +610,23 @@ extern "C" int omni_moe_gate_route(const void* x, int x_dtype, const void* gate_
   g.x = x; g.w = gate_w; g.T = T; g.H = H; g.E = E;
   g.slices_per_task = gate_slices_per_task(T, H, E);
   g.n_parts = (H / GATE_SLICE + g.slices_per_task - 1) / g.slices_per_task;
-  g.n_tt = (T + 63) / 64;
-  g.n_et = (E + 31) / 32;
+  const bool tile = g.slices_per_task == GATE_GROUP && T >= gate_tuning().tile_from;
+  g.n_tt = tile ? (T + GT_TOK - 1) / GT_TOK : (T + 63) / 64;
+  g.n_et = tile ? (E + GT_EXP - 1) / GT_EXP : (E + 31) / 32;
   g.partials = (float*)workspace;
   const int64_t tasks = (int64_t)g.n_parts * g.n_et * g.n_tt;
   if (tasks > 0x7fffffffLL) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: too many tasks");
-  dim3 grid((unsigned)tasks), block(64);
-  if (x_dtype == OMNI_DT_BF16 && w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_BF16, OMNI_DT_F32>), grid, block, 0, st, g);
-  else if (x_dtype == OMNI_DT_BF16) hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_BF16, OMNI_DT_BF16>), grid, block, 0, st, g);
-  else if (w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_F32, OMNI_DT_F32>), grid, block, 0, st, g);
-  else hipLaunchKernelGGL((gate_partial_kernel<OMNI_DT_F32, OMNI_DT_BF16>), grid, block, 0, st, g);
+  dim3 grid((unsigned)tasks), block(tile ? 256 : 64);
+#define GATE_LAUNCH(KERNEL)                                                                                   \
+  do {                                                                                                        \
+    if (x_dtype == OMNI_DT_BF16 && w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((KERNEL<OMNI_DT_BF16, OMNI_DT_F32>), grid, block, 0, st, g); \
+    else if (x_dtype == OMNI_DT_BF16) hipLaunchKernelGGL((KERNEL<OMNI_DT_BF16, OMNI_DT_BF16>), grid, block, 0, st, g);  \
+    else if (w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((KERNEL<OMNI_DT_F32, OMNI_DT_F32>), grid, block, 0, st, g);     \
+    else hipLaunchKernelGGL((KERNEL<OMNI_DT_F32, OMNI_DT_BF16>), grid, block, 0, st, g);                               \
+  } while (0)
+  if (tile) GATE_LAUNCH(gate_tile_kernel);
+  else GATE_LAUNCH(gate_partial_kernel);
+#undef GATE_LAUNCH
   OMNI_CHECK_LAUNCH("gate_partial");
   // few tokens: a block per token adds the parts up with its four wavefronts (the latency of one round of
   // loads instead of one per group); many tokens: a wavefront per token keeps every wavefront routing

@@ -55,6 +55,27 @@ def test_gate_logits_do_not_depend_on_the_batch(ops):
     assert _bits_equal(big[1000:1008], ref)
 
 
+@pytest.mark.parametrize("xdt,wdt", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                     (torch.float32, torch.float32), (torch.float32, torch.bfloat16)])
+def test_gate_logits_large_batch_kernel(ops, xdt, wdt):
+    """From 2048 tokens on a block of four wavefronts passes the operands through LDS (128 tokens x 64 experts
+    x a group of 8 slices).  Ragged token and expert tiles, a last group of 2 slices; the result must be the
+    bits of the small-batch kernel (64 tokens at a time) and of the oracle."""
+    g = gen(9)
+    T, H, E = 2048 + 77, 7168 + 256, 160
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(xdt).cuda()
+    w = (torch.randn(E, H, generator=g) * 0.02).to(wdt).cuda()
+    rb = wdt == torch.bfloat16
+    big = ops.gate_logits(x, w, round_logits_bf16=rb)
+    assert big.shape == (T, E)
+    for t0 in (0, 64, 1024, 2048, 2112):
+        small = ops.gate_logits(x[t0:t0 + 64].contiguous(), w, round_logits_bf16=rb)
+        assert _bits_equal(big[t0:t0 + 64], small), f"tokens {t0}.."
+    rows = torch.tensor([0, 63, 64, 127, 128, 2047, 2124])
+    ref = O.gate_logits_spec(x[rows.cuda()].cpu(), w.cpu(), round_bf16=rb)
+    assert _bits_equal(big[rows.cuda()], ref)
+
+
 @pytest.mark.parametrize("T,H,E", [(64, 7168, 256), (7, 1024, 64)])
 def test_gate_route_fused_equals_two_steps_and_oracle(ops, T, H, E):
     """omni_moe_gate_route = gate logits + the sigmoid/bias grouped router, one call: ids and weights equal
