@@ -48,9 +48,8 @@ __device__ __forceinline__ int source_row(const GemmArgs& a, int g, int r) {
   }
 }
 
-__device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float* __restrict__ wsc, int n, int row0,
-                                               int rbase, int nrows, const float* ts, v4i acc) {
-  const float ws = wsc[n];
+__device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float ws, int n, int row0, int rbase,
+                                               int nrows, const float* ts, v4i acc) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     int rr = rbase + i;
@@ -136,6 +135,12 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
   // way is then covered by the k loop instead of standing in front of the epilogue)
   if (threadIdx.x < 16 * MT)
     lds_ts[threadIdx.x] = ((int)threadIdx.x < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + threadIdx.x)] : 0.0f;
+
+  // the weight scales of this lane's output channels are requested here as well: asked for in the epilogue they
+  // would cost one more round trip through a saturated memory system at the end of every block's life
+  float wsv[NBF];
+#pragma unroll
+  for (int j = 0; j < NBF; ++j) wsv[j] = wsc[strip[j] * 16 + (lane & 15)];
 
   // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile, k-step w of
   // every chunk; rows past the end of the group alias the group's first row
@@ -231,7 +236,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
           for (int t = 0; t < NT; ++t) {
             const int n = strip[2 * t] * 16 + col;
-            const float wg = wsc[n], wu = wsc[I + n];
+            const float wg = wsv[2 * t], wu = wsv[2 * t + 1];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               if (rbase + i < nrows) {
@@ -272,7 +277,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
         for (int i = 0; i < 4; ++i) ts[i] = lds_ts[rbase + i];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsc, strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
+        for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsv[t], strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
       }
     }
   }
