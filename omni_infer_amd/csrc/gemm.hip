@@ -241,6 +241,158 @@ __device__ __forceinline__ void pipe_k_loop(const PipeCtx<WN>& c, int nk64, v4i*
   }
 }
 
+// =====================================================================================
+// Line layout of the activation operand (256 x 256 tiles, reduction length a multiple of 128).
+//   What bounds the tile kernel is the vector memory path of the CU (address unit and L1 busy all the time,
+//   the address unit held up by the L1 half of it), and a 16 row x 64 byte fragment is sixteen half cache
+//   lines: every line of an activation row was asked for twice, one k-step apart.  Here a load instruction
+//   fetches 8 rows x 128 bytes (whole lines; lane l: row l/8, one 16-byte piece) and an A stage holds two
+//   k-steps ("super-step"): 256 rows x 128 bytes = 32 KiB, three of them, next to the three 16 KiB B stages.
+//   global_load_lds stores a wavefront's 64 pieces linearly, so the bank swizzle is applied on the global
+//   side: slot q of row r holds piece q ^ f(r), f(r) = (r >> 1) & 7.  The 16 lanes of a quarter wavefront
+//   read one piece number of 16 consecutive rows: addresses 128 r + 16 (p ^ f(r)), which fall into 16
+//   different 16-byte bank groups.
+//   The instruction order of every half k-step is pinned: operands are read from LDS half a k-step before they
+//   are multiplied, into the registers the half step before has just released, and the reads and the loads
+//   that refill the ring are issued in the shadow of the running MFMAs.  The block barrier of a k-step sits
+//   between its halves.  sched_group_barrier masks: 0x008 MFMA, 0x020 vector memory read, 0x100 LDS read.
+// =====================================================================================
+struct LineCtx {
+  const int8_t* asrc[2][2];  // [k-step parity][i]: this lane's piece of its row, super-step 0
+  const int8_t* bsrc[2];
+  int w, lane;
+  int a_off[2][2];  // [k-step parity][half]: v4i index of the lane's A operand in a super-stage, row tile 0
+  int b_off[2];     // same for the two 32-channel tiles of the wavefront, half 0
+};
+constexpr int LINE_LPS = 4;  // loads per k-step per wavefront: 2 A instructions (8 rows each), 2 B fragments
+
+// the A loads of parity E fill rows [128 E, 128 E + 128) of a super-stage
+template <int E>
+__device__ __forceinline__ void line_load_a(const LineCtx& c, int ss, v4i* __restrict__ dst_a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    __builtin_amdgcn_global_load_lds(c.asrc[E][i] + (size_t)ss * 128, OMNI_LDS_PTR(dst_a + (E * 16 + 2 * c.w + i) * WAVE), 16, 0, 0);
+#endif
+}
+__device__ __forceinline__ void line_load_b(const LineCtx& c, int k, v4i* __restrict__ dst_b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    __builtin_amdgcn_global_load_lds(c.bsrc[i] + (size_t)k * 1024, OMNI_LDS_PTR(dst_b + (2 * c.w + i) * WAVE), 16, 0, 0);
+#endif
+}
+
+// operands of one half k-step of a wavefront that multiplies MTC row tiles of 32
+template <int MTC>
+struct LineOps { v4i a[MTC > 0 ? MTC : 1]; v4i b[2]; };
+
+template <int MTC, int E, int HALF>
+__device__ __forceinline__ void line_read(const LineCtx& c, const v4i* __restrict__ src_a, const v4i* __restrict__ src_b,
+                                          LineOps<MTC>& o) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) o.b[t] = src_b[c.b_off[t] + 32 * HALF];
+#pragma unroll
+  for (int mt = 0; mt < MTC; ++mt) o.a[mt] = src_a[c.a_off[E][HALF] + mt * 256];
+}
+
+template <int MTC>
+__device__ __forceinline__ void line_mfma(const LineOps<MTC>& o, v16i (&acc)[4][2]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int mt = 0; mt < MTC; ++mt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) acc[mt][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a[mt], o.b[t], acc[mt][t], 0, 0, 0);
+#endif
+}
+
+// pins the order of what is left of a half step: LDS reads two at a time, then the loads one at a time, each
+// group followed by one MFMA while there are MFMAs left, then the remaining MFMAs
+template <int D, int M, int V>
+__device__ __forceinline__ void line_pin() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if constexpr (D > 0) {
+    constexpr int n = D >= 2 ? 2 : 1;
+    __builtin_amdgcn_sched_group_barrier(0x100, n, 0);
+    if constexpr (M > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line_pin<D - n, (M > 0 ? M - 1 : 0), V>();
+  } else if constexpr (V > 0) {
+    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    if constexpr (M > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line_pin<0, (M > 0 ? M - 1 : 0), V - 1>();
+  } else if constexpr (M > 0) {
+    __builtin_amdgcn_sched_group_barrier(0x008, M, 0);
+  }
+#endif
+}
+
+// One k-step of parity E.  X holds the first-half operands of this k-step on entry and those of the next one
+// on exit.  After the barrier the B stage just read is refilled with k-step kb and this wavefront's share of
+// rows [128 E, 128 E + 128) of super-step ssa goes into `fill_a` (the super-stage read two super-steps ago).
+template <int MTC, int E>
+__device__ __forceinline__ void line_step(const LineCtx& c, int kb, int ssa, const v4i* __restrict__ cur_a,
+                                          v4i* __restrict__ cur_b, v4i* __restrict__ fill_a, const v4i* __restrict__ nxt_a,
+                                          const v4i* __restrict__ nxt_b, LineOps<MTC>& X, LineOps<MTC>& Y, v16i (&acc)[4][2]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if constexpr (MTC > 0) {
+    line_read<MTC, E, 1>(c, cur_a, cur_b, Y);
+    line_mfma<MTC>(X, acc);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line_pin<2 + MTC, 2 * MTC - 1, 0>();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // the next stage has landed (at most this wavefront's last k-step of loads is still in flight) and the
+  // wavefront has received everything it reads from the current one
+  __builtin_amdgcn_s_waitcnt((LINE_LPS & 0xF) | (0x7 << 4) | (0x0 << 8));
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  line_load_b(c, kb, cur_b);
+  line_load_a<E>(c, ssa, fill_a);
+  if constexpr (MTC > 0) {
+    line_read<MTC, 1 - E, 0>(c, nxt_a, nxt_b, X);
+    line_mfma<MTC>(Y, acc);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line_pin<2 + MTC, 2 * MTC - 1, LINE_LPS>();
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#endif
+}
+
+// the k loop: nk64 (even) k-steps; on entry super-steps 0 and 1 and k-steps 0 and 1 of B are on their way
+template <int MTC>
+__device__ __forceinline__ void line_k_loop(const LineCtx& c, int nk64, v4i* __restrict__ sa0, v4i* __restrict__ sa1,
+                                            v4i* __restrict__ sa2, v4i* __restrict__ sb0, v4i* __restrict__ sb1,
+                                            v4i* __restrict__ sb2, v16i (&acc)[4][2]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int last = nk64 - 1, last_ss = nk64 / 2 - 1;
+  LineOps<MTC> X, Y;
+  // super-step 0 and k-step 0 of B have landed: all loads but the last 6 (k-step 1 of B, super-step 1)
+  __builtin_amdgcn_s_waitcnt((6 & 0xF) | (0x7 << 4) | (0xF << 8));
+  __builtin_amdgcn_s_barrier();
+  line_load_b(c, min(2, last), sb2);
+  if constexpr (MTC > 0) line_read<MTC, 0, 0>(c, sa0, sb0, X);
+  __builtin_amdgcn_sched_barrier(0);
+  int k = 0;
+  for (; k + 6 <= nk64; k += 6) {
+    const int ss = k >> 1;
+    line_step<MTC, 0>(c, min(k + 3, last), min(ss + 2, last_ss), sa0, sb0, sa2, sa0, sb1, X, Y, acc);
+    line_step<MTC, 1>(c, min(k + 4, last), min(ss + 2, last_ss), sa0, sb1, sa2, sa1, sb2, X, Y, acc);
+    line_step<MTC, 0>(c, min(k + 5, last), min(ss + 3, last_ss), sa1, sb2, sa0, sa1, sb0, X, Y, acc);
+    line_step<MTC, 1>(c, min(k + 6, last), min(ss + 3, last_ss), sa1, sb0, sa0, sa2, sb1, X, Y, acc);
+    line_step<MTC, 0>(c, min(k + 7, last), min(ss + 4, last_ss), sa2, sb1, sa1, sa2, sb2, X, Y, acc);
+    line_step<MTC, 1>(c, min(k + 8, last), min(ss + 4, last_ss), sa2, sb2, sa1, sa0, sb0, X, Y, acc);
+  }
+  if (k < nk64) {  // two or four k-steps left; the rings are back at their first stages
+    line_step<MTC, 0>(c, last, last_ss, sa0, sb0, sa2, sa0, sb1, X, Y, acc);
+    line_step<MTC, 1>(c, last, last_ss, sa0, sb1, sa2, sa1, sb2, X, Y, acc);
+    if (k + 2 < nk64) {
+      line_step<MTC, 0>(c, last, last_ss, sa1, sb2, sa0, sa1, sb0, X, Y, acc);
+      line_step<MTC, 1>(c, last, last_ss, sa1, sb0, sa0, sa2, sb1, X, Y, acc);
+    }
+  }
+#endif
+}
+
 // 32x32 accumulator tile: lane l holds column l%32, rows 8*(i/4) + 4*(l/32) + i%4 for i = 0..15
 __device__ __forceinline__ int tile32_row(int lane, int i) { return 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3); }
 
@@ -380,14 +532,18 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
 // per CU (a third fewer operand bytes through the vector memory path per MFMA).
 // BF (GEMM1 only): round gate, up and their product to bf16 (the numerics of the reference's
 // unfused bf16 path); a template parameter so that the fp32 path carries none of that arithmetic.
-template <int KIND, int WN, bool BF>
+// LINES (WN = 4, reduction length a multiple of 128): the line layout of the activation operand and the
+// pinned k loop above; otherwise fragments of 16 rows x 64 bytes and the loop the compiler schedules.
+template <int KIND, int WN, bool BF, bool LINES>
 __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int BM = 256;
   constexpr int NBS = 4 * WN;             // B strips per stage
   constexpr int GS = 2 * WN;              // KIND 1: gate strips per block
   constexpr int AP = PipeCtx<WN>::A_PER_WAVE;
-  __shared__ v4i sa0[16 * WAVE], sa1[16 * WAVE], sa2[16 * WAVE];
+  static_assert(!LINES || WN == 4, "the line layout is written for the 256 x 256 tile");
+  constexpr int A_STAGE = LINES ? 32 * WAVE : 16 * WAVE;  // v4i per A stage: 256 rows x 128 or x 64 bytes
+  __shared__ v4i sa0[A_STAGE], sa1[A_STAGE], sa2[A_STAGE];
   __shared__ v4i sb0[NBS * WAVE], sb1[NBS * WAVE], sb2[NBS * WAVE];
   __shared__ __attribute__((aligned(16))) float row_scale[BM];  // activation scale of every row of the block
 
@@ -425,7 +581,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     int left = 0;
     if (a.tail_part != nullptr && a.tile_slots > 0) {
       left = n_real % a.tile_slots;
-      if (left > 0 && 2 * left <= a.tile_slots) split = min(min(a.tile_split_max, a.tile_slots / left), nk_all);
+      if (left > 0 && 2 * left <= a.tile_slots) split = min(min(a.tile_split_max, a.tile_slots / left), LINES ? nk_all / 2 : nk_all);
       if (split < 2) { split = 1; left = 0; }
     }
     int id = (int)blockIdx.x;
@@ -458,8 +614,10 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   RowBlock rb;
   if (!row_blocks_find(scan, a.offsets, a.G, a.extra_rows, BM, by, rb)) return;
   // this block's k-steps [k_first, k_first + nk64)
-  const int k_first = (tail_tile >= 0) ? share * nk_all / split : 0;
-  const int k_end = (tail_tile >= 0) ? (share + 1) * nk_all / split : nk_all;
+  // (shares of the line layout begin and end on whole super-steps of 128)
+  constexpr int KU = LINES ? 2 : 1;
+  const int k_first = (tail_tile >= 0) ? share * (nk_all / KU) / split * KU : 0;
+  const int k_end = (tail_tile >= 0) ? (share + 1) * (nk_all / KU) / split * KU : nk_all;
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int nk64 = k_end - k_first;
   const int I = (KIND == 1) ? a.N / 2 : 0;
@@ -472,34 +630,72 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     if constexpr (KIND == 1) return (j < GS) ? bx * GS + j : I / 16 + bx * GS + (j - GS);
     else return bx * NBS + j;
   };
-#pragma unroll
-  for (int i = 0; i < AP; ++i) {
-    int rr = (AP * w + i) * 16 + (lane & 15);
-    if (rr >= nrows) rr = 0;  // rows past the end alias the first row; their results are not stored
-    c.asrc[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k_first * 64 + (lane >> 4) * 16;
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-    c.bsrc[i] = wbase + ((size_t)strip_of(2 * w + i) * nk_all + k_first) * 1024 + lane * 16;
-  // the first two k-steps are requested as soon as their addresses exist; everything else the block
-  // has to set up overlaps with their flight
   const int last = nk64 - 1;
-  pipe_load<WN>(c, 0, sa0, sb0);
-  pipe_load<WN>(c, min(1, last), sa1, sb1);
-  // per-row activation scales go to LDS once (read back in the epilogue, after many barriers)
-  for (int r = threadIdx.x; r < BM; r += 128 * WN) {
-    row_scale[r] = (r < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + r)] : 0.0f;
-  }
-  // operand addressing of the 32x32x32 form (see the header comment)
+  // operand addressing of the 32x32x32 form (see the header comment): B, and A in the fragment layout
   const int in_pair = ((lane & 31) >> 4) * WAVE + (lane & 15) + 16 * (lane >> 5);
-  c.a_off = (wm * 8) * WAVE + in_pair;
   // wavefront column wn: KIND 1: gate tile = strips {2wn, 2wn+1}, up tile = strips {GS+2wn, GS+2wn+1};
   //                      KIND 2: tiles = strips {4wn, 4wn+1} and {4wn+2, 4wn+3}
   int tile_strip0[2];
   if constexpr (KIND == 1) { tile_strip0[0] = 2 * wn; tile_strip0[1] = GS + 2 * wn; }
   else { tile_strip0[0] = 4 * wn; tile_strip0[1] = 4 * wn + 2; }
+  // 32-row tiles of this wavefront that hold rows of the block
+  c.mt_count = min(4, max(0, (nrows - wm * 128 + 31) / 32));
+  LineCtx lc;
+  if constexpr (LINES) {
+    lc.w = w;
+    lc.lane = lane;
 #pragma unroll
-  for (int t = 0; t < 2; ++t) c.b_off[t] = tile_strip0[t] * WAVE + in_pair;
+    for (int e = 0; e < 2; ++e)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int r_tile = (e * 16 + 2 * w + i) * 8 + (lane >> 3);  // the row of the tile this lane fetches a piece of
+        int rr = r_tile;
+        if (rr >= nrows) rr = 0;  // rows past the end alias the first row; their results are not stored
+        const int piece = (lane & 7) ^ ((r_tile >> 1) & 7);
+        lc.asrc[e][i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k_first * 64 + piece * 16;
+      }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      lc.bsrc[i] = wbase + ((size_t)strip_of(2 * w + i) * nk_all + k_first) * 1024 + lane * 16;
+    // the first two super-steps of A and k-steps of B are requested as soon as their addresses exist (in the
+    // order the first barrier of the k loop counts on); everything else the block sets up overlaps with them
+    const int last_ss = nk64 / 2 - 1;
+    line_load_a<0>(lc, 0, sa0);
+    line_load_a<1>(lc, 0, sa0);
+    line_load_b(lc, 0, sb0);
+    line_load_b(lc, min(1, last), sb1);
+    line_load_a<0>(lc, min(1, last_ss), sa1);
+    line_load_a<1>(lc, min(1, last_ss), sa1);
+    const int r32 = lane & 31;
+    const int gx = (lane >> 5) ^ ((r32 >> 1) & 7);
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) lc.a_off[e][h] = (wm * 128 + r32) * 8 + ((4 * e + 2 * h) ^ gx);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) lc.b_off[t] = tile_strip0[t] * WAVE + in_pair;
+  } else {
+#pragma unroll
+    for (int i = 0; i < AP; ++i) {
+      int rr = (AP * w + i) * 16 + (lane & 15);
+      if (rr >= nrows) rr = 0;  // rows past the end alias the first row; their results are not stored
+      c.asrc[i] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k_first * 64 + (lane >> 4) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      c.bsrc[i] = wbase + ((size_t)strip_of(2 * w + i) * nk_all + k_first) * 1024 + lane * 16;
+    // the first two k-steps are requested as soon as their addresses exist; everything else the block
+    // has to set up overlaps with their flight
+    pipe_load<WN>(c, 0, sa0, sb0);
+    pipe_load<WN>(c, min(1, last), sa1, sb1);
+    c.a_off = (wm * 8) * WAVE + in_pair;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) c.b_off[t] = tile_strip0[t] * WAVE + in_pair;
+  }
+  // per-row activation scales go to LDS once (read back in the epilogue, after many barriers)
+  for (int r = threadIdx.x; r < BM; r += 128 * WN) {
+    row_scale[r] = (r < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + r)] : 0.0f;
+  }
 
   v16i acc[4][2];
 #pragma unroll
@@ -509,10 +705,21 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
 
-  // wavefronts whose 128 rows all exist take the loop without tests
-  c.mt_count = min(4, max(0, (nrows - wm * 128 + 31) / 32));
-  if (c.mt_count == 4) pipe_k_loop<WN, false>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
-  else pipe_k_loop<WN, true>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
+  if constexpr (LINES) {
+    // one instantiation of the pinned loop per number of row tiles; a wavefront without rows only takes
+    // part in the loads and the barriers
+    switch (c.mt_count) {
+      case 4: line_k_loop<4>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      case 3: line_k_loop<3>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      case 2: line_k_loop<2>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      case 1: line_k_loop<1>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      default: line_k_loop<0>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+    }
+  } else {
+    // wavefronts whose 128 rows all exist take the loop without tests
+    if (c.mt_count == 4) pipe_k_loop<WN, false>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
+    else pipe_k_loop<WN, true>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
+  }
   // no LDS traffic may still be in flight when the block's LDS is handed to the next block
   __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));  // vmcnt(0)
 
@@ -623,12 +830,13 @@ struct Plan {
 //   OMNI_MOE_G1 / _G2      "mt,nt,d[,S]" of the stream kernel of GEMM1 / GEMM2; a combination that is not
 //                          compiled in is refused here, with a message, and the default is used
 //   OMNI_MOE_TILE_WN       2: tile kernel of 256 x 128 instead of 256 x 256
+//   OMNI_MOE_TILE_LINES    0: the 256 x 256 tile kernel keeps the fragment layout of the activation operand
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
 //   OMNI_MOE_EQUAL_PROGRESS 0: the stream kernel of GEMM1 leaves the issue priority of its wavefronts alone
 struct Tuning {
-  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1;
+  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
   bool have[3] = {false, false, false};
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
@@ -646,6 +854,7 @@ const Tuning& tuning() {
     r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
     r.rowq = geti("OMNI_MOE_ROWQ", 0);
     r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
+    r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
     for (int kind = 1; kind <= 2; ++kind) {
       const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
       const char* e = getenv(name);
@@ -745,6 +954,9 @@ void launch_stream(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st)
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }
 
+// the line layout of the activation operand needs whole super-steps of 128 (OMNI_MOE_TILE_LINES=0: never)
+bool tile_lines(int Kdim) { return tuning().tile_lines && Kdim % 128 == 0; }
+
 // wavefront columns of the large tile: 4 (256 channels per block) when the channel count allows, else 2
 int tile_wn(int kind, int units) {
   const int wide = (kind == 1) ? 8 : 16;  // units per 256-channel block
@@ -808,12 +1020,15 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, si
   }
   dim3 grid((unsigned)nblocks), block(128 * wn);
   const bool bfi = KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE);
-  if (wn == 4) {
-    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((gemm_pipe<KIND, 4, false>), grid, block, 0, st, a);
+  if (wn == 4 && tile_lines(a.Kdim)) {
+    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_pipe<KIND, 4, false, true>), grid, block, 0, st, a);
+  } else if (wn == 4) {
+    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1, false>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_pipe<KIND, 4, false, false>), grid, block, 0, st, a);
   } else {
-    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 2, KIND == 1>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((gemm_pipe<KIND, 2, false>), grid, block, 0, st, a);
+    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 2, KIND == 1, false>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((gemm_pipe<KIND, 2, false, false>), grid, block, 0, st, a);
   }
 }
 
@@ -972,7 +1187,10 @@ extern "C" int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extr
   if (M_cap < 0 || I <= 0 || H <= 0 || G < 0 || (kind == 1 && (T <= 0 || K <= 0))) OMNI_FAIL(OMNI_E_INVALID, "gemm_kernel_name: bad sizes");
   const Plan p = (kind == 1) ? make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap)
                              : make_plan<2>((int)M_cap, 1, G, extra_rows, I, H, M_cap);
-  if (p.tile) snprintf(buf, buf_bytes, "gemm_pipe<%d,%d>", kind, tile_wn(kind, kind == 1 ? 2 * I / 32 : H / 16));
+  if (p.tile) {
+    const int wn = tile_wn(kind, kind == 1 ? 2 * I / 32 : H / 16);
+    snprintf(buf, buf_bytes, "gemm_pipe<%d,%d,%s>", kind, wn, (wn == 4 && tile_lines(kind == 1 ? H : I)) ? "lines" : "frags");
+  }
   else snprintf(buf, buf_bytes, "gemm_stream<%d,%d,%d,%d>", kind, p.mt, p.nt, p.d);
   return OMNI_OK;
 }
