@@ -288,6 +288,92 @@ __device__ __forceinline__ bool row_blocks_find(const RowBlockScan& s, const int
   rb.nrows = __builtin_amdgcn_readlane(nrows, owner);
   return true;
 }
+// The same row blocks numbered by weight: first the heavy blocks of all groups in group order (full blocks, and
+// last blocks with more than `light_max` rows), then the light last blocks of the groups that have one.  A
+// kernel whose blocks cost the same from light_max + 1 rows on can then deal out equal work first and keep the
+// cheap blocks for the end.
+struct RowBlockKinds {
+  int start, c;              // Gt <= 64: this lane's group (first row, rows)
+  int incl_h, nh;            // inclusive prefix and count of the heavy blocks of this lane's group(s)
+  int incl_l, nl;            // same for the light blocks
+  int total_h, total_l;
+  bool small;
+};
+__device__ __forceinline__ int heavy_blocks(int c, int BM, int light_max) { return c / BM + ((c % BM) > light_max); }
+__device__ __forceinline__ int light_blocks(int c, int BM, int light_max) { return (c % BM) > 0 && (c % BM) <= light_max; }
+__device__ __forceinline__ RowBlockKinds row_block_kinds_scan(const int32_t* __restrict__ offsets, int G, int extra_rows,
+                                                              int BM, int light_max) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int Gt = G + (extra_rows > 0 ? 1 : 0);
+  RowBlockKinds s{};
+  s.small = Gt <= WAVE;
+  if (s.small) {
+    if (lane < Gt) {
+      s.start = offsets[lane < G ? lane : G];
+      s.c = (lane < G) ? (offsets[lane + 1] - s.start) : extra_rows;
+    }
+    s.nh = heavy_blocks(s.c, BM, light_max);
+    s.nl = light_blocks(s.c, BM, light_max);
+  } else {
+    const int per = (Gt + WAVE - 1) / WAVE;
+    for (int j = 0; j < per; ++j) {
+      const int g = lane * per + j;
+      if (g < Gt) {
+        const int c = (g < G) ? (offsets[g + 1] - offsets[g]) : extra_rows;
+        s.nh += heavy_blocks(c, BM, light_max);
+        s.nl += light_blocks(c, BM, light_max);
+      }
+    }
+  }
+  s.incl_h = wave_incl_scan_dpp_i(s.nh);
+  s.incl_l = wave_incl_scan_dpp_i(s.nl);
+  s.total_h = __builtin_amdgcn_readlane(s.incl_h, WAVE - 1);
+  s.total_l = __builtin_amdgcn_readlane(s.incl_l, WAVE - 1);
+  return s;
+}
+// heavy block b (light == false) or light block b; b must be in range
+__device__ __forceinline__ void row_block_kinds_find(const RowBlockKinds& s, const int32_t* __restrict__ offsets, int G,
+                                                     int extra_rows, int BM, int light_max, bool light, int b, RowBlock& rb) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int incl = light ? s.incl_l : s.incl_h;
+  const int excl = incl - (light ? s.nl : s.nh);
+  const uint64_t owner_mask = __ballot(b >= excl && b < incl);
+  const int owner = __ffsll((unsigned long long)owner_mask) - 1;
+  if (s.small) {
+    const int o_start = __builtin_amdgcn_readlane(s.start, owner);
+    const int o_c = __builtin_amdgcn_readlane(s.c, owner);
+    const int o_excl = __builtin_amdgcn_readlane(excl, owner);
+    rb.group = owner;
+    const int first = light ? o_c / BM * BM : (b - o_excl) * BM;  // row of the group the block starts at
+    rb.row0 = o_start + first;
+    rb.nrows = min(BM, o_c - first);
+    return;
+  }
+  const int Gt = G + (extra_rows > 0 ? 1 : 0);
+  const int per = (Gt + WAVE - 1) / WAVE;
+  int grp = -1, row0 = 0, nrows = 0;
+  if (lane == owner) {
+    int acc = excl;
+    for (int j = 0; j < per; ++j) {
+      const int g = lane * per + j;
+      if (g >= Gt) break;
+      const int start = offsets[g < G ? g : G];
+      const int c = (g < G) ? (offsets[g + 1] - start) : extra_rows;
+      const int n = light ? light_blocks(c, BM, light_max) : heavy_blocks(c, BM, light_max);
+      if (b < acc + n) {
+        const int first = light ? c / BM * BM : (b - acc) * BM;
+        grp = g;
+        row0 = start + first;
+        nrows = min(BM, c - first);
+        break;
+      }
+      acc += n;
+    }
+  }
+  rb.group = __builtin_amdgcn_readlane(grp, owner);
+  rb.row0 = __builtin_amdgcn_readlane(row0, owner);
+  rb.nrows = __builtin_amdgcn_readlane(nrows, owner);
+}
 __device__ __forceinline__ bool find_row_block(const int32_t* __restrict__ offsets, int G, int extra_rows, int BM,
                                                int b, RowBlock& rb) {
   const RowBlockScan s = row_blocks_scan(offsets, G, extra_rows, BM);

@@ -554,13 +554,19 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   c.wn = c.w % WN;
   const int lane = c.lane, w = c.w, wm = c.wm, wn = c.wn;
   // ---- which tile, and which share of its reduction
-  // Real tiles (row blocks that exist x column tiles) get the ids [0, n_real) in three runs:
+  // A block's time is set by the wavefronts of its first 128 rows, so a row block costs the same from 97
+  // rows on ("heavy"); only the last blocks of groups with at most 96 rows left are cheaper ("light").
+  // Real tiles (row blocks that exist x column tiles) get the ids [0, n_real): first the tiles of the heavy
+  // row blocks, then those of the light ones, each set in three runs:
   //   A: whole patches of TILE_PR row blocks x tile_pc column tiles, in rounds of 8 dealt to the 8 XCDs
-  //      (workgroups go to the XCDs, each with its own L2, round-robin by their linear id, so the
-  //      tiles an XCD runs together share their row panels and, inside an expert, their weight
-  //      panels in that L2);
+  //      (workgroups go to the XCDs, each with its own L2 and its own dispatcher, round-robin by their
+  //      linear id, so the tiles an XCD runs together share their row panels and, inside an expert,
+  //      their weight panels in that L2);
   //   B: the whole patches that do not fill a round of 8, one after the other;
   //   C: the row blocks past the last whole patch row, row by row.
+  // Every XCD works through its own ids in order and nothing moves work between XCDs, so the heavy tiles,
+  // which all cost the same, are dealt out evenly by count and the cheap tiles fill in at the end (with
+  // light blocks scattered among the heavy ones the XCDs finished 8 % apart at 8192 tokens).
   // With n_real tiles on `tile_slots` block slots the last n_real % tile_slots tiles would run alone
   // on a nearly idle chip.  When they are at most half a round, each of them is split S ways along the
   // reduction: the tile's own block takes the first share, helper blocks with ids past n_real the
@@ -568,16 +574,15 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // counter adds the others' to its own (integer sums: the order cannot matter) and runs the
   // epilogue.  Nobody waits for anybody.
   constexpr int TILE_PR = 4;
-  const RowBlockScan scan = row_blocks_scan(a.offsets, a.G, a.extra_rows, BM);
+  constexpr int LIGHT_MAX = 96;
+  const RowBlockKinds scan = row_block_kinds_scan(a.offsets, a.G, a.extra_rows, BM, LIGHT_MAX);
   const int nk_all = a.Kdim / 64;
   int bx, by, split = 1, share = 0, tail_tile = -1;
+  bool light;
   {
     const int gx = a.tile_gx, pc = a.tile_pc, npc = gx / pc, per_patch = TILE_PR * pc;
-    const int RB = scan.total;
-    const int n_real = RB * gx;
-    const int bulk_rows = RB / TILE_PR * TILE_PR;
-    const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
-    const int nA = patches8 * per_patch, nB = (patches - patches8) * per_patch;
+    const int n_heavy = scan.total_h * gx;
+    const int n_real = (scan.total_h + scan.total_l) * gx;
     int left = 0;
     if (a.tail_part != nullptr && a.tile_slots > 0) {
       left = n_real % a.tile_slots;
@@ -594,25 +599,32 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     } else if (split > 1 && id >= n_real - left) {
       tail_tile = id - (n_real - left);
     }
-    if (id < nA + nB) {
+    light = id >= n_heavy;
+    const int t = light ? id - n_heavy : id;              // id inside the set
+    const int RB = light ? scan.total_l : scan.total_h;   // row blocks of the set
+    const int bulk_rows = RB / TILE_PR * TILE_PR;
+    const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
+    const int nA = patches8 * per_patch, nB = (patches - patches8) * per_patch;
+    if (t < nA + nB) {
       int patch, q;
-      if (id < nA) {
-        const int xcd = id & 7, j = id >> 3;
-        patch = (j / per_patch) * 8 + xcd;
+      if (t < nA) {
+        // the tiles of a patch are 8 ids apart: one XCD runs them all
+        const int j = t >> 3;
+        patch = (j / per_patch) * 8 + (t & 7);
         q = j % per_patch;
       } else {
-        patch = patches8 + (id - nA) / per_patch;
-        q = (id - nA) % per_patch;
+        patch = patches8 + (t - nA) / per_patch;
+        q = (t - nA) % per_patch;
       }
       by = (patch / npc) * TILE_PR + q / pc;
       bx = (patch % npc) * pc + q % pc;
     } else {
-      by = bulk_rows + (id - nA - nB) / gx;
-      bx = (id - nA - nB) % gx;
+      by = bulk_rows + (t - nA - nB) / gx;
+      bx = (t - nA - nB) % gx;
     }
   }
   RowBlock rb;
-  if (!row_blocks_find(scan, a.offsets, a.G, a.extra_rows, BM, by, rb)) return;
+  row_block_kinds_find(scan, a.offsets, a.G, a.extra_rows, BM, LIGHT_MAX, light, by, rb);
   // this block's k-steps [k_first, k_first + nk64)
   // (shares of the line layout begin and end on whole super-steps of 128)
   constexpr int KU = LINES ? 2 : 1;
