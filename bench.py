@@ -40,7 +40,8 @@ INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/cl
 # be read from inside a timed run, so these are values of record, labelled with the summary they come from.
 RECORDED_TRAFFIC = {
     ("decode", "gemm1"): (987_888_000, "profiles/decode_gemm1_hbm_traffic.txt"),
-    ("prefill", "gemm1"): (7_283_159_000, "profiles/prefill_gemm1_hbm_traffic.txt"),
+    ("prefill", "gemm1"): (5_613_418_000, "profiles/prefill_gemm1_hbm_traffic.txt"),
+    ("prefill", "gemm2"): (5_043_485_000, "profiles/prefill_gemm1_hbm_traffic.txt"),
 }
 
 SHAPES = {
