@@ -213,11 +213,20 @@ size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int 
 /*
  * Which GEMM kernel the two entry points above launch for a call of these sizes (kind 1: GEMM1 with the
  * arguments of omni_moe_gemm1_swiglu_quant; kind 2: GEMM2, T and K unused), written to buf as the kernel's
- * template name, e.g. "gemm_stream<1,2,1,4>" or "gemm_pipe<2,4>".  A diagnostic for benchmarks and profiles
+ * template name, e.g. "gemm_stream<1,2,1,4>" or "gemm_pipe<2,4,lines>" (256 x 64*4 tile, line layout of the
+ * activation operand; "frags": fragment layout).  A diagnostic for benchmarks and profiles
  * (no counterpart in the reference, whose kernels are chosen inside the closed operators).
  */
 int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, char* buf,
                               size_t buf_bytes);
+
+/*
+ * The OMNI_MOE_* tuning variables (kernel choice, tile shape, split tiles ...) are read from the environment
+ * once, at the first GEMM call of the process.  This reads them again: for tests and tuning runs that change
+ * them inside one process.  Not to be called while another thread launches GEMMs.  No counterpart in the
+ * reference.
+ */
+void omni_moe_reload_tuning(void);
 
 /*
  * Diagnostic (no counterpart in the reference): the sustained rate of v_mfma_i32_32x32x32_i8 on given operand

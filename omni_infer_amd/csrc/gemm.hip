@@ -853,36 +853,39 @@ struct Tuning {
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
 bool stream_variant_exists(int kind, int mt, int nt, int d);
-const Tuning& tuning() {
-  static const Tuning t = [] {
-    Tuning r;
-    auto geti = [](const char* name, int dflt) {
-      const char* v = getenv(name);
-      return v ? atoi(v) : dflt;
-    };
-    r.force_kernel = geti("OMNI_MOE_FORCE_KERNEL", 0);
-    r.tile_wn = geti("OMNI_MOE_TILE_WN", 4);
-    r.tile_tail = geti("OMNI_MOE_TILE_TAIL", 1);
-    r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
-    r.rowq = geti("OMNI_MOE_ROWQ", 0);
-    r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
-    r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
-    for (int kind = 1; kind <= 2; ++kind) {
-      const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
-      const char* e = getenv(name);
-      if (!e) continue;
-      int mt = 0, nt = 0, d = 0, S = 0;
-      if (sscanf(e, "%d,%d,%d,%d", &mt, &nt, &d, &S) >= 3 && stream_variant_exists(kind, mt, nt, d)) {
-        r.have[kind] = true;
-        r.mt[kind] = mt; r.nt[kind] = nt; r.d[kind] = d; r.S[kind] = S;
-      } else {
-        fprintf(stderr, "omni_moe: %s=\"%s\" names no compiled stream kernel; ignored\n", name, e);
-      }
+Tuning read_tuning() {
+  Tuning r;
+  auto geti = [](const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : dflt;
+  };
+  r.force_kernel = geti("OMNI_MOE_FORCE_KERNEL", 0);
+  r.tile_wn = geti("OMNI_MOE_TILE_WN", 4);
+  r.tile_tail = geti("OMNI_MOE_TILE_TAIL", 1);
+  r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
+  r.rowq = geti("OMNI_MOE_ROWQ", 0);
+  r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
+  r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
+  for (int kind = 1; kind <= 2; ++kind) {
+    const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
+    const char* e = getenv(name);
+    if (!e) continue;
+    int mt = 0, nt = 0, d = 0, S = 0;
+    if (sscanf(e, "%d,%d,%d,%d", &mt, &nt, &d, &S) >= 3 && stream_variant_exists(kind, mt, nt, d)) {
+      r.have[kind] = true;
+      r.mt[kind] = mt; r.nt[kind] = nt; r.d[kind] = d; r.S[kind] = S;
+    } else {
+      fprintf(stderr, "omni_moe: %s=\"%s\" names no compiled stream kernel; ignored\n", name, e);
     }
-    return r;
-  }();
+  }
+  return r;
+}
+// read at the first GEMM call of the process; omni_moe_reload_tuning() reads the environment again
+Tuning& tuning_store() {
+  static Tuning t = read_tuning();
   return t;
 }
+const Tuning& tuning() { return tuning_store(); }
 
 // the compiled (KIND, MT, NT, D) combinations of gemm_stream
 #define OMNI_STREAM_VARIANTS(X)                                                        \
@@ -1192,6 +1195,8 @@ extern "C" size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t 
   Plan p = make_plan<2>((int)M_cap, 1, G, extra_rows, I, H, M_cap);
   return p.tile ? TILE_TAIL_BYTES : 0;
 }
+
+extern "C" void omni_moe_reload_tuning(void) { tuning_store() = read_tuning(); }
 
 extern "C" int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I,
                                          char* buf, size_t buf_bytes) {

@@ -189,10 +189,13 @@ def _grouped_case(T, K, n_local, E, H, I, seed, lo=0):
     (700, 2, 3, 3, 1024, 512, 2),       # tile kernel, 24 tiles per GEMM: each tile's reduction is shared by four blocks
     (520, 1, 1, 1, 2048, 1024, 2),      # one group of three row blocks: 24 / 96 tiles, split four ways / two ways
 ])
-def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, monkeypatch):
+def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, tuning):
     from omni_infer_amd import _lib as L
     if force:
-        monkeypatch.setenv("OMNI_MOE_FORCE_KERNEL", str(force))
+        tuning(OMNI_MOE_FORCE_KERNEL=force)
+        want = {1: "gemm_stream", 2: "gemm_pipe"}[force]
+        for kind in (1, 2):   # the forced kernel is the one the library will launch
+            assert ops.gemm_kernel_name(kind, T, K, n_local, 0, T * K, H, I).startswith(want)
     lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 20 + T)
     d = lay.to_device()
     out_ref, st = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (0, n_local),
@@ -221,7 +224,7 @@ def test_gemm1_gemm2_stages(ops, T, K, n_local, E, H, I, force, monkeypatch):
     _eq(out, out_ref, "combined output")
 
 
-def test_split_tiles_equal_unsplit(ops, monkeypatch):
+def test_split_tiles_equal_unsplit(ops, tuning):
     """Tiles of the last partial round share their reduction between blocks (integer partial sums, the
     last block to arrive adds them): the results are the same bits as with the sharing switched off."""
     from omni_infer_amd import _lib as L
@@ -229,10 +232,9 @@ def test_split_tiles_equal_unsplit(ops, monkeypatch):
     lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 77)
     d = lay.to_device()
     p = ops.moe_permute(ids.cuda(), 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
-    monkeypatch.setenv("OMNI_MOE_FORCE_KERNEL", "2")
     got = {}
     for tail in ("1", "0"):
-        monkeypatch.setenv("OMNI_MOE_TILE_TAIL", tail)
+        tuning(OMNI_MOE_FORCE_KERNEL=2, OMNI_MOE_TILE_TAIL=tail)
         for rep in range(10):   # repeated launches reuse the same scratch and counters
             h_q, h_s, acc1 = ops.grouped_gemm1_swiglu_quant(xq.cuda(), xs.cuda(), p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K,
                                                             d["w13"], d["s13"], p.offsets, H, I, T * K, want_acc=True)
@@ -246,6 +248,73 @@ def test_split_tiles_equal_unsplit(ops, monkeypatch):
     for a, b, what in zip(got["1"], got["0"], ("h_q", "h_s", "acc1", "rows", "acc2")):
         m = int(p.offsets[-1])
         assert torch.equal(a[:m], b[:m]), f"{what}: split and unsplit tiles differ"
+
+
+def _tile_outputs(ops, lay_dev, xq, xs, p, K, H, I, M_cap):
+    from omni_infer_amd import _lib as L
+    h_q, h_s, acc1 = ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, lay_dev["w13"],
+                                                    lay_dev["s13"], p.offsets, H, I, M_cap, want_acc=True)
+    out = [h_q, h_s, acc1]
+    for dt in (torch.float32, torch.bfloat16):
+        rows, acc2 = ops.grouped_gemm2_dequant(h_q, h_s, lay_dev["w2"], lay_dev["s2"], p.offsets, H, I, out_dtype=dt,
+                                               want_acc=True)
+        out += [rows, acc2]
+    return [t.cpu() for t in out]
+
+
+@pytest.mark.parametrize("T,K,n_local,E,H,I", [
+    (700, 2, 3, 3, 1024, 512),     # a few row blocks per group, partial last blocks, split tiles
+    (1500, 4, 6, 8, 1536, 768),    # light (at most 96 rows) and heavy last blocks mixed, reduction of 12 and 6 super-steps
+])
+def test_tile_layouts_give_the_same_bits(ops, tuning, T, K, n_local, E, H, I):
+    """The tile kernel has two layouts of the activation operand in LDS (whole 128-byte lines with the pinned
+    k loop, the default where it applies, and 16-row fragments) and two tile widths: all of them give the bits
+    of the oracle."""
+    from omni_infer_amd import _lib as L
+    lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 300 + T)
+    d = lay.to_device()
+    _, st = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (0, n_local),
+                                              return_stages=True)
+    m = int(st["counts"].sum())
+    p = ops.moe_permute(ids.cuda(), 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    M_cap = T * K
+    seen = {}
+    for tag, env in (("lines", dict(OMNI_MOE_TILE_LINES=1, OMNI_MOE_TILE_WN=4)),
+                     ("frags", dict(OMNI_MOE_TILE_LINES=0, OMNI_MOE_TILE_WN=4)),
+                     ("narrow", dict(OMNI_MOE_TILE_LINES=1, OMNI_MOE_TILE_WN=2))):
+        tuning(OMNI_MOE_FORCE_KERNEL=2, **env)
+        name = ops.gemm_kernel_name(1, T, K, n_local, 0, M_cap, H, I)
+        assert name == {"lines": "gemm_pipe<1,4,lines>", "frags": "gemm_pipe<1,4,frags>", "narrow": "gemm_pipe<1,2,frags>"}[tag]
+        seen[tag] = _tile_outputs(ops, d, xq.cuda(), xs.cuda(), p, K, H, I, M_cap)
+    h_q, h_s, acc1 = seen["lines"][:3]
+    _eq(acc1[:m], st["acc1"], "GEMM1 int32 accumulators")
+    _eq(h_s[:m], st["h_s"], "stage-2 scales")
+    _eq(h_q[:m], st["h_q"], "stage-2 int8 activations")
+    _eq(seen["lines"][4][:m], st["acc2"], "GEMM2 int32 accumulators")
+    for tag in ("frags", "narrow"):
+        for a, b, what in zip(seen[tag], seen["lines"], ("h_q", "h_s", "acc1", "rows f32", "acc2", "rows bf16", "acc2")):
+            assert torch.equal(a[:m], b[:m]), f"{what}: {tag} differs from the line layout"
+
+
+def test_tile_kernel_odd_number_of_k_steps(ops, tuning):
+    """A reduction length that is a multiple of 64 but not of 128 (17 k-steps) takes the fragment layout of the
+    tile kernel; GEMM2 of this shape (1088 channels: no whole tile) goes to the stream kernel."""
+    from omni_infer_amd import _lib as L
+    T, K, n_local, E, H, I = 600, 2, 3, 3, 1088, 512
+    tuning(OMNI_MOE_FORCE_KERNEL=2)
+    assert ops.gemm_kernel_name(1, T, K, n_local, 0, T * K, H, I) == "gemm_pipe<1,4,frags>"
+    lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 411)
+    d = lay.to_device()
+    out_ref, st = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (0, n_local),
+                                                    return_stages=True)
+    m = int(st["counts"].sum())
+    p = ops.moe_permute(ids.cuda(), 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    got = _tile_outputs(ops, d, xq.cuda(), xs.cuda(), p, K, H, I, T * K)
+    _eq(got[2][:m], st["acc1"], "GEMM1 int32 accumulators")
+    _eq(got[0][:m], st["h_q"], "stage-2 int8 activations")
+    _eq(got[4][:m], st["acc2"], "GEMM2 int32 accumulators")
+    out = ops.moe_combine(got[3].cuda(), w.cuda(), p.src_to_dst, L.OMNI_IDX_TOKEN_MAJOR, L.OMNI_ORDER_SLOT)
+    _eq(out, out_ref, "combined output")
 
 
 def test_combine_k_order_with_skip(ops):
