@@ -429,6 +429,50 @@ def bench_calib(args):
         res[f"vendor_int_mm_{tag}_pops"] = 2.0 * M * K * N / (ms * 1e-3) / 1e15
         res[f"vendor_int_mm_{tag}_us"] = ms * 1e3
         del a, b
+    # the library's own tile kernels at the prefill shape, once on the real operands and once on zeros: the
+    # same instruction stream at the clock the chip grants each kind of data
+    from omni_infer_amd import hip_ops as ops
+    cfg = SHAPES["prefill"]
+    T, H, I, K, n_local = cfg["T"], cfg["H"], cfg["I"], cfg["K"], cfg["n_local"]
+    ws = WeightSet(cfg, 100, dev)
+    ws.drop_ckpt()
+    x, logits, bias = make_inputs(cfg, dev)
+    w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
+    p = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
+    M_cap = T * K + T
+    xq, xs = ops.npu_dynamic_quant(x)
+    g1_ws = torch.zeros(lib.omni_moe_gemm1_workspace_bytes(T, K, n_local, T, M_cap, H, I), dtype=torch.uint8, device=dev)
+    hq = torch.empty(M_cap, I, dtype=torch.int8, device=dev)
+    hs = torch.empty(M_cap, dtype=torch.float32, device=dev)
+    rows = torch.empty(M_cap, H, dtype=torch.float32, device=dev)
+
+    def g1(flags=L.OMNI_GEMM1_NO_REQUANT):
+        ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, ws.w13, ws.s13, p.offsets, H, I,
+                                       M_cap, extra=(ws.sh13, ws.sh_s13), extra_rows=T, flags=flags, workspace=g1_ws,
+                                       out=(hq, hs))
+
+    def g2():
+        ops.grouped_gemm2_dequant(hq, hs, ws.w2, ws.s2, p.offsets, H, I, out_dtype=torch.float32,
+                                  extra=(ws.sh2, ws.sh_s2), extra_rows=T, out=rows, workspace=g1_ws)
+
+    g1(0)   # real int8 rows for GEMM2
+    res["tile_kernels"] = {"gemm1": ops.gemm_kernel_name(1, T, K, n_local, T, M_cap, H, I),
+                           "gemm2": ops.gemm_kernel_name(2, T, K, n_local, T, M_cap, H, I), "rows": M_cap}
+    res["tile_gemm1_real_operands_us"] = ev_ms(g1, 10) * 1e3
+    res["tile_gemm2_real_operands_us"] = ev_ms(g2, 10) * 1e3
+    xq.zero_()
+    hq.zero_()
+    res["tile_gemm1_zero_activations_us"] = ev_ms(g1, 10) * 1e3
+    res["tile_gemm2_zero_activations_us"] = ev_ms(g2, 10) * 1e3
+    for t in (ws.w13, ws.sh13, ws.w2, ws.sh2):
+        t.zero_()
+    res["tile_gemm1_zero_operands_us"] = ev_ms(g1, 10) * 1e3
+    res["tile_gemm2_zero_operands_us"] = ev_ms(g2, 10) * 1e3
+    ops1, ops2 = 2.0 * M_cap * H * 2 * I, 2.0 * M_cap * I * H
+    for k in ("real_operands", "zero_operands"):
+        res[f"tile_gemm1_{k}_pops"] = ops1 / (res[f"tile_gemm1_{k}_us"] * 1e-6) / 1e15
+        res[f"tile_gemm2_{k}_pops"] = ops2 / (res[f"tile_gemm2_{k}_us"] * 1e-6) / 1e15
+    del ws, xq, hq, rows, g1_ws
     src = torch.ones(1 << 30, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
     ms = ev_ms(lambda: dst.copy_(src), 10)
