@@ -265,6 +265,8 @@ def _tile_outputs(ops, lay_dev, xq, xs, p, K, H, I, M_cap):
 @pytest.mark.parametrize("T,K,n_local,E,H,I", [
     (700, 2, 3, 3, 1024, 512),     # a few row blocks per group, partial last blocks, split tiles
     (1500, 4, 6, 8, 1536, 768),    # light (at most 96 rows) and heavy last blocks mixed, reduction of 12 and 6 super-steps
+    (900, 2, 2, 2, 256, 128),      # the shortest reductions: two super-steps and one
+    (2100, 1, 1, 1, 384, 640),     # one group of nine row blocks; three and five super-steps (loop remainders of 0, 2 and 4 k-steps)
 ])
 def test_tile_layouts_give_the_same_bits(ops, tuning, T, K, n_local, E, H, I):
     """The tile kernel has two layouts of the activation operand in LDS (whole 128-byte lines with the pinned
