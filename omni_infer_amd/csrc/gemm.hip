@@ -846,7 +846,8 @@ struct Plan {
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
-//   OMNI_MOE_EQUAL_PROGRESS 0: the stream kernel of GEMM1 leaves the issue priority of its wavefronts alone
+//   OMNI_MOE_EQUAL_PROGRESS bit 0: the stream kernel of GEMM1 lowers the issue priority of its wavefronts as they
+//                          advance (default 1), bit 1: that of GEMM2 too (measured slower in every geometry)
 struct Tuning {
   int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
   bool have[3] = {false, false, false};
@@ -912,11 +913,11 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
   const int64_t per = (G > 0) ? avg : extra_rows;
   Plan p{};
   p.per = per;
-  // Measured on the DeepSeek-V3 shape (32 routed groups + the shared one): up to 48 expected rows per
+  // Measured on the DeepSeek-V3 shape (32 routed groups + the shared one): up to 56 expected rows per
   // routed group the stream kernel wins (row blocks of 64 rows from 25 expected rows on, so that
   // nearly every group is one block and its weights are read once; the shared group then takes a few
   // blocks and re-reads its 3 % of the bytes); above that the tile kernel does.
-  p.tile = (G > 0) ? per > 48 : per > 128;
+  p.tile = (G > 0) ? per > 56 : per > 128;
   const Tuning& tn = tuning();
   const int force = tn.force_kernel;
   if (force == 1) p.tile = false;
@@ -964,7 +965,7 @@ void launch_stream(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st)
   int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
   // GEMM1 (every block resident at once, long streams) gains from equal progress; GEMM2 (three rounds of short
   // blocks, where the older round should finish first and make room) loses by it: measured 84.4 -> 87.6 us
-  a.equal_progress = (KIND == 1 && a.S == 1) ? tuning().equal_progress : 0;
+  a.equal_progress = (KIND == 1 && a.S == 1) ? (tuning().equal_progress & 1) : (tuning().equal_progress >> 1);
   dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks, (unsigned)a.S), block(256);
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }

@@ -123,7 +123,7 @@ class DeepseekMoE(nn.Module):
                 if lin.quant_method is not None:
                     lin.quant_method.process_weights_after_loading(lin)
 
-    def _route(self, hidden_states):
+    def _route(self, hidden_states, attn_metadata=None):
         """``self.gate.forward(hidden_states.float())`` + ``FusedMoE.select_experts`` (deepseek_moe.py:253-256,
         329-333).  The fused body makes both in one library call on the tokens as they are; the
         operator-by-operator body keeps the reference's two steps.  Same bits either way."""
@@ -139,7 +139,9 @@ class DeepseekMoE(nn.Module):
                 hidden_states, router_logits, e.top_k, e.use_grouped_topk, e.renormalize, e.topk_group,
                 e.num_expert_group, e.custom_routing_function, e.scoring_func, e.e_score_correction_bias,
                 self.routed_scaling_factor, layer=e)
-        return topk_weights, e.apply_expert_load_balance(topk_ids=topk_ids)
+        # the decode paths hand the forced-balance ids of the attention metadata on (deepseek_moe.py:343, :399)
+        best = getattr(getattr(attn_metadata, "decode", None), "best_topk", None)
+        return topk_weights, e.apply_expert_load_balance(topk_ids=topk_ids, best_topk_ids=best)
 
     def forward(self, hidden_states: torch.Tensor, residual: torch.Tensor, attn_metadata, layer_id: int = 0,
                 next_attention_weights: Optional[dict] = None):
@@ -149,7 +151,7 @@ class DeepseekMoE(nn.Module):
         same_width = (self.shared_experts is None or
                       self.shared_experts.down_proj.input_size == self.experts.intermediate_size_per_partition)
         if self.fused and allgather_ep and same_width and self.quant_symbol:
-            return self._forward_fused(hidden_states), residual
+            return self._forward_fused(hidden_states, attn_metadata), residual
         if isinstance(hidden_states, dict):
             hidden_states = hidden_states["x"]
         return self._forward_norm_ops(hidden_states, attn_metadata), residual
@@ -164,20 +166,20 @@ class DeepseekMoE(nn.Module):
             x_in, pertoken_scale = ops.npu_dynamic_quant(hidden_states)
         else:
             x_in, pertoken_scale = hidden_states, None
-        topk_weights, topk_ids = self._route(hidden_states)
+        topk_weights, topk_ids = self._route(hidden_states, attn_metadata)
         final = self.experts(hidden_states=x_in, topk_weights=topk_weights, topk_ids=topk_ids,
                              pertoken_scale=pertoken_scale, attn_metadata=attn_metadata)
         if shared_output is not None:
             final = final + shared_output
         return final
 
-    def _forward_fused(self, hidden_states):
+    def _forward_fused(self, hidden_states, attn_metadata=None):
         # a dict from RMSNorm.forward_moe_input carries the tokens already quantised
         x_int8 = pertoken_scale = None
         if isinstance(hidden_states, dict):
             x_int8, pertoken_scale = hidden_states["x_int8"], hidden_states["pertoken_scale"]
             hidden_states = hidden_states["x"]
-        topk_weights, topk_ids = self._route(hidden_states)
+        topk_weights, topk_ids = self._route(hidden_states, attn_metadata)
         e = self.experts
         lo = self.global_rank * self.local_expert_num
         shared = None

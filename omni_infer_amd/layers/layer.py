@@ -10,6 +10,8 @@ from __future__ import annotations
 
 from typing import Callable, Optional
 
+import os
+
 import torch
 
 from .. import hip_ops as ops
@@ -53,6 +55,7 @@ class FusedMoE(torch.nn.Module):
         self.num_expert_group = num_expert_group
         self.topk_group = topk_group
         self.custom_routing_function = custom_routing_function
+        self.is_prefill_instance = os.environ.get("ROLE", "") == "prefill"   # layer.py:228
         if quant_config is None:
             raise NotImplementedError("only the W8A8 quantised MoE method is built (no bf16 expert path)")
         self.quant_method = quant_config.get_quant_method(self, prefix)
@@ -69,10 +72,20 @@ class FusedMoE(torch.nn.Module):
             raise ValueError("Only softmax scoring function is supported for non-grouped topk.")
 
     def apply_expert_load_balance(self, topk_ids: torch.Tensor, best_topk_ids: Optional[torch.Tensor] = None):
-        """layer.py:273-299: identity here (no placement planner, no forced balance)."""
+        """layer.py:273-299: the placement planner's remap when a planner was given (none is built here), then the
+        forced balance of the ``best_ep`` flag: a prefill instance (``ROLE=prefill``) replaces the routing by
+        the ids 0..255 dealt round robin, eight per token (the reference hard-codes 256 experts and top-8 at
+        :291-292); elsewhere the caller's ``best_topk_ids`` are taken when given."""
         if self.planner is not None:
             _, topk_ids, _ = self.planner.plan(layer_idx_moe=self.moe_layer_idx, tokens=None, token_expert_ids=topk_ids,
                                                token_expert_scores=None, expert_mapping=self.expert_mapping)
+        if model_extra_config.operator_opt_config.best_ep:
+            if self.is_prefill_instance:
+                t = (topk_ids.shape[0] * 8) // 256
+                topk_ids = torch.arange(256, device=topk_ids.device, dtype=torch.int32).unsqueeze(0).repeat(t + 1, 1) \
+                    .view(-1, 8)[:topk_ids.shape[0]]
+            elif best_topk_ids is not None:
+                topk_ids = best_topk_ids
         return topk_ids
 
     @staticmethod

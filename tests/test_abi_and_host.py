@@ -174,6 +174,31 @@ def test_weight_loader_places_shards():
         distributed.set_virtual_ep(1, 0)
 
 
+def test_forced_expert_balance(monkeypatch):
+    """apply_expert_load_balance with the best_ep flag (reference layer.py:288-297): a prefill instance deals the
+    256 expert ids round robin, eight per token, whatever the router chose; a decode instance takes the caller's
+    ids when it is given some; without the flag the routing passes through."""
+    from omni_infer_amd import config
+    from omni_infer_amd.layers.layer import FusedMoE
+    from omni_infer_amd.quantization.compressed_tensors import AscendCompressedTensorsConfig
+    ids = torch.randint(0, 256, (70, 8), dtype=torch.int32)
+    best = torch.randint(0, 256, (70, 8), dtype=torch.int32)
+    try:
+        m = FusedMoE(8, 2, 128, 64, params_dtype=torch.bfloat16, quant_config=AscendCompressedTensorsConfig())
+        assert torch.equal(m.apply_expert_load_balance(ids, best), ids)
+        config.update_model_extra_config(best_ep=True)
+        assert torch.equal(m.apply_expert_load_balance(ids, best), best)      # decode instance
+        assert torch.equal(m.apply_expert_load_balance(ids), ids)
+        monkeypatch.setenv("ROLE", "prefill")
+        p = FusedMoE(8, 2, 128, 64, params_dtype=torch.bfloat16, quant_config=AscendCompressedTensorsConfig())
+        got = p.apply_expert_load_balance(ids, best)
+        assert got.shape == ids.shape and got.dtype == torch.int32
+        assert torch.equal(got.reshape(-1), torch.arange(70 * 8, dtype=torch.int32) % 256)
+        assert int(torch.bincount(got.reshape(-1).long(), minlength=256).max()) <= 70 * 8 // 256 + 1
+    finally:
+        config.update_model_extra_config(best_ep=False)
+
+
 def test_product_never_touches_the_oracle():
     """The shipped package must not import, call or read anything under oracle/."""
     pkg = os.path.join(ROOT, "omni_infer_amd")
