@@ -421,3 +421,43 @@ def test_layer_entry_shape_sweep(ops, T, K, n_local, E, H, I, shared, seed):
         assert "multiple of 256" in str(e) or "not divisible" in str(e), str(e)
         return
     _eq(out, want, f"layer output T={T} K={K} n_local={n_local}/{E} H={H} I={I} shared={shared}")
+
+
+# ------------------------------------------------------------------ seeded sweep over tile-kernel shapes
+def _tile_sweep_cases():
+    """14 seeded shapes that the 256 x 256 tile kernel with the line layout serves: hundreds to thousands of
+    tokens, skewed routing (full, heavy, light and empty row blocks side by side), widths whose reductions
+    are 1 to 6 super-steps of 128, with and without the shared expert."""
+    g = gen(777)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    cases = []
+    for n in range(14):
+        E = r(1, 10)
+        n_local = r(1, E)
+        K = r(1, min(E, 3))
+        T = [600, 900, 1300, 2200, 3100, 777, 1025][n % 7]
+        cases.append((T, K, n_local, E, 256 * r(1, 3), 128 * r(1, 3), bool(n & 1), n))
+    return cases
+
+
+@pytest.mark.parametrize("T,K,n_local,E,H,I,shared,seed", _tile_sweep_cases())
+def test_layer_entry_tile_sweep(ops, tuning, T, K, n_local, E, H, I, shared, seed):
+    tuning(OMNI_MOE_FORCE_KERNEL=2)
+    assert ops.gemm_kernel_name(1, T, K, n_local, T if shared else 0, T * K + (T if shared else 0), H, I) == "gemm_pipe<1,4,lines>"
+    assert ops.gemm_kernel_name(2, T, K, n_local, T if shared else 0, T * K + (T if shared else 0), H, I) == "gemm_pipe<2,4,lines>"
+    g = gen(7000 + seed)
+    lay = Layer(n_local, H, I, seed=7000 + seed, shared=shared)
+    x = tokens(T, H, 8000 + seed)
+    pop = torch.randn(E, generator=g) * 1.5          # a few popular experts, a few nearly empty ones
+    ids = (torch.rand(T, E, generator=g) + pop * 0.4).argsort(dim=1, descending=True)[:, :K].to(torch.int32)
+    w = torch.rand(T, K, generator=g)
+    lo = int(torch.randint(0, E - n_local + 1, (1,), generator=g))
+    xq, xs = O.dynamic_quant(x)
+    want = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (lo, lo + n_local))
+    if shared:
+        want = (want.float() + O.shared_expert_mlp(x, *lay.shared).float()).to(torch.bfloat16)
+    d = lay.to_device()
+    sh = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]) if shared else None
+    out = ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), lo, lo + n_local, d["w13"], d["s13"], d["w2"], d["s2"],
+                             sh, H=H, I=I)
+    _eq(out, want, f"layer output T={T} K={K} n_local={n_local}/{E} H={H} I={I} shared={shared}")
