@@ -283,18 +283,6 @@ __device__ __forceinline__ void line_load_b(const LineCtx& c, int k, v4i* __rest
 #endif
 }
 
-// what a tile's k loop expects to be on its way when it starts: super-steps 0 and 1 of A, k-steps 0 and 1 of B
-__device__ __forceinline__ void line_first_loads(const LineCtx& c, int nk64, v4i* __restrict__ sa0, v4i* __restrict__ sa1,
-                                                 v4i* __restrict__ sb0, v4i* __restrict__ sb1) {
-  const int last = nk64 - 1, last_ss = nk64 / 2 - 1;
-  line_load_a<0>(c, 0, sa0);
-  line_load_a<1>(c, 0, sa0);
-  line_load_b(c, 0, sb0);
-  line_load_b(c, min(1, last), sb1);
-  line_load_a<0>(c, min(1, last_ss), sa1);
-  line_load_a<1>(c, min(1, last_ss), sa1);
-}
-
 // operands of one half k-step of a wavefront that multiplies MTC row tiles of 32
 template <int MTC>
 struct LineOps { v4i a[MTC > 0 ? MTC : 1]; v4i b[2]; };
@@ -372,17 +360,14 @@ __device__ __forceinline__ void line_step(const LineCtx& c, int kb, int ssa, con
 
 // the k loop: nk64 (even) k-steps; on entry super-steps 0 and 1 and k-steps 0 and 1 of B are on their way
 template <int MTC>
-__device__ __forceinline__ void line_k_loop(const LineCtx& c, int nk64, bool drain, v4i* __restrict__ sa0,
-                                            v4i* __restrict__ sa1, v4i* __restrict__ sa2, v4i* __restrict__ sb0,
-                                            v4i* __restrict__ sb1, v4i* __restrict__ sb2, v16i (&acc)[4][2]) {
+__device__ __forceinline__ void line_k_loop(const LineCtx& c, int nk64, v4i* __restrict__ sa0, v4i* __restrict__ sa1,
+                                            v4i* __restrict__ sa2, v4i* __restrict__ sb0, v4i* __restrict__ sb1,
+                                            v4i* __restrict__ sb2, v16i (&acc)[4][2]) {
 #if defined(__HIP_DEVICE_COMPILE__)
   const int last = nk64 - 1, last_ss = nk64 / 2 - 1;
   LineOps<MTC> X, Y;
-  // super-step 0 and k-step 0 of B have landed: all loads but the last 6 (k-step 1 of B, super-step 1).  With
-  // `drain` (the second tile of a block: the stores of the first tile's epilogue were issued after these loads,
-  // and stores and loads share the counter) everything is waited for.
-  if (drain) __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));
-  else __builtin_amdgcn_s_waitcnt((6 & 0xF) | (0x7 << 4) | (0xF << 8));
+  // super-step 0 and k-step 0 of B have landed: all loads but the last 6 (k-step 1 of B, super-step 1)
+  __builtin_amdgcn_s_waitcnt((6 & 0xF) | (0x7 << 4) | (0xF << 8));
   __builtin_amdgcn_s_barrier();
   line_load_b(c, min(2, last), sb2);
   if constexpr (MTC > 0) line_read<MTC, 0, 0>(c, sa0, sb0, X);
@@ -418,20 +403,10 @@ __device__ __forceinline__ int tile32_row(int lane, int i) { return 8 * (i >> 2)
 // once fall into disjoint banks) and stored as whole 128-byte lines.
 constexpr int TILE_OUT_PITCH_DW = 48;
 #define TILE_STAGE_DWORDS (32 * TILE_OUT_PITCH_DW)  // staging dwords of one wavefront
-// the weight scales of the two channels a lane holds (asked for ahead of the epilogue: see tile_epilogue_after_loads)
-template <int KIND, int WN>
-__device__ __forceinline__ void tile_weight_scales(const float* __restrict__ wsc, int lane, int wn, int bx, int I,
-                                                   float (&wsc_g)[2]) {
-  const int c32 = lane & 31;
-  const int n0 = (KIND == 1) ? (bx * 2 * WN + 2 * wn) * 16 + c32 : (bx * 4 * WN + 4 * wn) * 16 + c32;
-  wsc_g[0] = wsc[n0];
-  wsc_g[1] = wsc[(KIND == 1) ? I + n0 : n0 + 32];
-}
-
 template <int KIND, int WN, bool BF>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][2], const float* row_scale,
                                               uint32_t* stage32, int lane, int wm, int wn, int bx, int row0,
-                                              int nrows, const float (&wsc_g)[2], int I) {
+                                              int nrows, const float* __restrict__ wsc, int I) {
   constexpr int NBS = 4 * WN;
   constexpr int GS = 2 * WN;
   // ---- epilogue, one 32-row tile at a time
@@ -439,6 +414,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
   constexpr int OUT_PITCH_DW = TILE_OUT_PITCH_DW;
   const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
   constexpr bool bf = BF;
+  float wsc_g[2];
   int ncol[2];
   if constexpr (KIND == 1) {
     ncol[0] = (bx * GS + 2 * wn) * 16 + c32;
@@ -447,6 +423,8 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
     ncol[0] = (bx * NBS + 4 * wn) * 16 + c32;
     ncol[1] = ncol[0] + 32;
   }
+  wsc_g[0] = wsc[ncol[0]];
+  wsc_g[1] = wsc[ncol[1]];
   if (bf16_out) {
     if constexpr (KIND == 2) {
       const int odd = c32 & 1;
@@ -550,29 +528,6 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
   }
 }
 
-// The epilogue of a tile that is followed by another one of the same block (line layout): the next tile's first
-// operands are requested first.  One function with every LDS pointer __restrict__, so that the compiler sees
-// that the row scales the epilogue reads do not alias the stages those loads write, and does not wait for the
-// loads in front of its first LDS read.
-template <int KIND, int WN, bool BF>
-__device__ __forceinline__ void tile_epilogue_after_loads(const GemmArgs& a, v16i (&acc)[4][2], const float* __restrict__ row_scale,
-                                                          uint32_t* stage32, int lane, int wm, int wn, int bx, int row0, int nrows,
-                                                          const float* __restrict__ wsc, int I, const LineCtx& lc, int nk64,
-                                                          v4i* __restrict__ sa0, v4i* __restrict__ sa1, v4i* __restrict__ sb0,
-                                                          v4i* __restrict__ sb1) {
-  // the weight scales are asked for ahead of the operand loads: loads come back in order, so the epilogue's wait
-  // for the scales does not wait for the operands
-  float wsc_g[2];
-  tile_weight_scales<KIND, WN>(wsc, lane, wn, bx, I, wsc_g);
-  __builtin_amdgcn_sched_barrier(0);
-  line_first_loads(lc, nk64, sa0, sa1, sb0, sb1);
-  // all but the 12 operand loads just issued: the scales are there (said explicitly: left to itself the compiler
-  // waits for every load in front of the first use of a scale)
-  __builtin_amdgcn_s_waitcnt((12 & 0xF) | (0x7 << 4) | (0xF << 8));
-  __builtin_amdgcn_sched_barrier(0);
-  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wm, wn, bx, row0, nrows, wsc_g, I);
-}
-
 // WN = 2: 256 threads, tile 256 x 128, two blocks per CU.  WN = 4: 512 threads, tile 256 x 256, one block
 // per CU (a third fewer operand bytes through the vector memory path per MFMA).
 // BF (GEMM1 only): round gate, up and their product to bf16 (the numerics of the reference's
@@ -618,49 +573,34 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // others.  Every share stores its int32 partial accumulators; whoever arrives last at the tile's
   // counter adds the others' to its own (integer sums: the order cannot matter) and runs the
   // epilogue.  Nobody waits for anybody.
-  const int TILE_PR = a.tile_pr;
+  constexpr int TILE_PR = 4;
   constexpr int LIGHT_MAX = 96;
   const RowBlockKinds scan = row_block_kinds_scan(a.offsets, a.G, a.extra_rows, BM, LIGHT_MAX);
   const int nk_all = a.Kdim / 64;
   int bx, by, split = 1, share = 0, tail_tile = -1;
-  bool light, pair = false;
+  bool light;
   {
     const int gx = a.tile_gx, pc = a.tile_pc, npc = gx / pc, per_patch = TILE_PR * pc;
     const int n_heavy = scan.total_h * gx;
     const int n_real = (scan.total_h + scan.total_l) * gx;
-    // Two tiles per block (line layout, large launches; the host sets tile_pair and an even tile_pc): the tiles
-    // of run A of the heavy set are taken in pairs of neighbouring column tiles of one row block.  The second
-    // tile's first operands are requested before the first tile's epilogue, so its set-up and first wait
-    // disappear.  Pair blocks come first, the remaining tiles follow one per block.
-    int n_pairs = 0;
-    if (LINES && a.tile_pair) {
-      const int bulk_h = scan.total_h / TILE_PR * TILE_PR;
-      n_pairs = (bulk_h / TILE_PR * npc) / 8 * 8 * per_patch / 2;
-    }
-    const int n_blocks = n_real - n_pairs;
     int left = 0;
     if (a.tail_part != nullptr && a.tile_slots > 0) {
-      left = n_blocks % a.tile_slots;
-      if (left > 0 && 2 * left <= a.tile_slots && left <= n_blocks - n_pairs)
-        split = min(min(a.tile_split_max, a.tile_slots / left), LINES ? nk_all / 2 : nk_all);
+      left = n_real % a.tile_slots;
+      if (left > 0 && 2 * left <= a.tile_slots) split = min(min(a.tile_split_max, a.tile_slots / left), LINES ? nk_all / 2 : nk_all);
       if (split < 2) { split = 1; left = 0; }
     }
     int id = (int)blockIdx.x;
-    if (id >= n_blocks) {
-      const int h = id - n_blocks;
+    if (id >= n_real) {
+      const int h = id - n_real;
       if (split == 1 || h >= left * (split - 1)) return;
       tail_tile = h / (split - 1);
       share = 1 + h % (split - 1);
-      id = n_blocks - left + tail_tile;
-    } else if (split > 1 && id >= n_blocks - left) {
-      tail_tile = id - (n_blocks - left);
+      id = n_real - left + tail_tile;
+    } else if (split > 1 && id >= n_real - left) {
+      tail_tile = id - (n_real - left);
     }
-    pair = id < n_pairs;
-    // tile id in the order of the two sets: a pair block takes the tiles tid and tid + 8 (the next tile of the
-    // same XCD: the next column of the same row block, tile_pc being even)
-    const int tid = pair ? ((id >> 3) << 4) + (id & 7) : id + n_pairs;
-    light = tid >= n_heavy;
-    const int t = light ? tid - n_heavy : tid;            // id inside the set
+    light = id >= n_heavy;
+    const int t = light ? id - n_heavy : id;              // id inside the set
     const int RB = light ? scan.total_l : scan.total_h;   // row blocks of the set
     const int bulk_rows = RB / TILE_PR * TILE_PR;
     const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
@@ -731,7 +671,13 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
       lc.bsrc[i] = wbase + ((size_t)strip_of(2 * w + i) * nk_all + k_first) * 1024 + lane * 16;
     // the first two super-steps of A and k-steps of B are requested as soon as their addresses exist (in the
     // order the first barrier of the k loop counts on); everything else the block sets up overlaps with them
-    line_first_loads(lc, nk64, sa0, sa1, sb0, sb1);
+    const int last_ss = nk64 / 2 - 1;
+    line_load_a<0>(lc, 0, sa0);
+    line_load_a<1>(lc, 0, sa0);
+    line_load_b(lc, 0, sb0);
+    line_load_b(lc, min(1, last), sb1);
+    line_load_a<0>(lc, min(1, last_ss), sa1);
+    line_load_a<1>(lc, min(1, last_ss), sa1);
     const int r32 = lane & 31;
     const int gx = (lane >> 5) ^ ((r32 >> 1) & 7);
 #pragma unroll
@@ -763,112 +709,77 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     row_scale[r] = (r < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + r)] : 0.0f;
   }
 
-  const int ncols = (LINES && pair) ? 2 : 1;
   v16i acc[4][2];
-  for (int ci = 0; ci < ncols; ++ci) {
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
+
+  if constexpr (LINES) {
+    // one instantiation of the pinned loop per number of row tiles; a wavefront without rows only takes
+    // part in the loads and the barriers
+    switch (c.mt_count) {
+      case 4: line_k_loop<4>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      case 3: line_k_loop<3>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      case 2: line_k_loop<2>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      case 1: line_k_loop<1>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      default: line_k_loop<0>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+    }
+  } else {
+    // wavefronts whose 128 rows all exist take the loop without tests
+    if (c.mt_count == 4) pipe_k_loop<WN, false>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
+    else pipe_k_loop<WN, true>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
+  }
+  // no LDS traffic may still be in flight when the block's LDS is handed to the next block
+  __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));  // vmcnt(0)
+
+  // ---- epilogue (the stage buffers are free now: the bf16 rows of GEMM2 are staged there, two
+  // wavefronts per buffer)
+  __syncthreads();  // every wavefront is done reading the last stage; the row scales written at the start are visible
+  if (tail_tile >= 0) {
+    // one share of a split tile: publish the partial sums, count in, and only the last one goes on
+    __shared__ int s_last;
+    constexpr int WAVE_INTS = 8 * 16 * WAVE;           // accumulator words of one wavefront
+    constexpr int TILE_INTS = 2 * WN * WAVE_INTS;
+    // Hand-over between the shares of a tile (their blocks may run on different XCDs, each with its own
+    // L2).  Every wavefront stores its partial sums, all wavefronts meet at the block barrier, then one
+    // thread counts in with a device-scope acquire-release add: the release half makes every store
+    // that happened before it (the barrier orders the other wavefronts' stores before it) visible to
+    // the device before the counter moves, and whoever reads the final count has, through the acquire
+    // half and the chain of adds on the same counter, all other shares' stores visible to its block
+    // after the second barrier.  No share ever waits for another.
+    int32_t* mine = a.tail_part + ((size_t)tail_tile * split + share) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
+      if (mt < c.mt_count) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
-
-    if constexpr (LINES) {
-      // one instantiation of the pinned loop per number of row tiles; a wavefront without rows only takes
-      // part in the loads and the barriers
-      switch (c.mt_count) {
-        case 4: line_k_loop<4>(lc, nk64, ci > 0, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-        case 3: line_k_loop<3>(lc, nk64, ci > 0, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-        case 2: line_k_loop<2>(lc, nk64, ci > 0, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-        case 1: line_k_loop<1>(lc, nk64, ci > 0, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-        default: line_k_loop<0>(lc, nk64, ci > 0, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+          for (int i = 0; i < 16; ++i) mine[((mt * 2 + t) * 16 + i) * WAVE] = acc[mt][t][i];
       }
-    } else {
-      // wavefronts whose 128 rows all exist take the loop without tests
-      if (c.mt_count == 4) pipe_k_loop<WN, false>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
-      else pipe_k_loop<WN, true>(c, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc);
-    }
-    // no LDS traffic may still be in flight when the block's LDS is handed to the next block
-    __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));  // vmcnt(0)
-
-    // ---- epilogue (the stage buffers are free now: the bf16 rows of GEMM2 are staged there, two
-    // wavefronts per buffer)
-    __syncthreads();  // every wavefront is done reading the last stage; the row scales written at the start are visible
-    // First row, row count and lane are made opaque per tile: everything after the k loop that is computed from
-    // them (row indices, bounds tests, the store addresses of the epilogue and of the split-tile hand-over) would
-    // otherwise be worked out ahead of the first k loop, for both tiles at once, and spilled over it.
-    int row0_now = row0, nrows_now = nrows, lane_now = lane;
-    asm volatile("" : "+s"(row0_now), "+s"(nrows_now), "+v"(lane_now));
-    if (tail_tile >= 0) {
-      // one share of a split tile: publish the partial sums, count in, and only the last one goes on
-      __shared__ int s_last;
-      constexpr int WAVE_INTS = 8 * 16 * WAVE;           // accumulator words of one wavefront
-      constexpr int TILE_INTS = 2 * WN * WAVE_INTS;
-      // Hand-over between the shares of a tile (their blocks may run on different XCDs, each with its own
-      // L2).  Every wavefront stores its partial sums, all wavefronts meet at the block barrier, then one
-      // thread counts in with a device-scope acquire-release add: the release half makes every store
-      // that happened before it (the barrier orders the other wavefronts' stores before it) visible to
-      // the device before the counter moves, and whoever reads the final count has, through the acquire
-      // half and the chain of adds on the same counter, all other shares' stores visible to its block
-      // after the second barrier.  No share ever waits for another.
-      int32_t* mine = a.tail_part + ((size_t)tail_tile * split + share) * TILE_INTS + (size_t)w * WAVE_INTS + lane_now;
+    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
+    __syncthreads();
+    if (threadIdx.x == 0)
+      s_last = (__hip_atomic_fetch_add(a.tail_cnt + tail_tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == split - 1);
+    __syncthreads();
+    if (!s_last) return;
+    for (int s2 = 0; s2 < split; ++s2) {
+      if (s2 == share) continue;
+      const int32_t* theirs = a.tail_part + ((size_t)tail_tile * split + s2) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
         if (mt < c.mt_count) {
 #pragma unroll
           for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) mine[((mt * 2 + t) * 16 + i) * WAVE] = acc[mt][t][i];
+            for (int i = 0; i < 16; ++i) acc[mt][t][i] += theirs[((mt * 2 + t) * 16 + i) * WAVE];
         }
-      __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
-      __syncthreads();
-      if (threadIdx.x == 0)
-        s_last = (__hip_atomic_fetch_add(a.tail_cnt + tail_tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == split - 1);
-      __syncthreads();
-      if (!s_last) return;
-      for (int s2 = 0; s2 < split; ++s2) {
-        if (s2 == share) continue;
-        const int32_t* theirs = a.tail_part + ((size_t)tail_tile * split + s2) * TILE_INTS + (size_t)w * WAVE_INTS + lane_now;
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-          if (mt < c.mt_count) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-              for (int i = 0; i < 16; ++i) acc[mt][t][i] += theirs[((mt * 2 + t) * 16 + i) * WAVE];
-          }
-      }
-    }
-    uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
-    // a second tile follows (the next column tile of the same rows): its weight pointers are the first tile's
-    // moved on by one column tile, and its first operands are requested before this tile's epilogue, except
-    // where the epilogue stages bf16 rows in the buffers they land in
-    const bool more = ci + 1 < ncols;
-    bool done = false;
-    if constexpr (LINES) {
-      if (more) {
-        const size_t col_step = (size_t)((KIND == 1) ? GS : NBS) * nk_all * 1024;
-        lc.bsrc[0] += col_step;
-        lc.bsrc[1] += col_step;
-        if (KIND == 2 && a.out_dtype == OMNI_DT_BF16) {
-          float wsc_g[2];
-          tile_weight_scales<KIND, WN>(wsc, lane_now, wn, bx + ci, I, wsc_g);
-          tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane_now, wm, wn, bx + ci, row0_now, nrows_now, wsc_g, I);
-          __syncthreads();  // every wavefront has read its staged rows back
-          line_first_loads(lc, nk64, sa0, sa1, sb0, sb1);
-        } else {
-          tile_epilogue_after_loads<KIND, WN, BF>(a, acc, row_scale, stage32, lane_now, wm, wn, bx + ci, row0_now, nrows_now,
-                                                  wsc, I, lc, nk64, sa0, sa1, sb0, sb1);
-        }
-        done = true;
-      }
-    }
-    if (!done) {
-      float wsc_g[2];
-      tile_weight_scales<KIND, WN>(wsc, lane_now, wn, bx + ci, I, wsc_g);
-      tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane_now, wm, wn, bx + ci, row0_now, nrows_now, wsc_g, I);
     }
   }
+  uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
+  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wm, wn, bx, row0, nrows, wsc, I);
 #endif
 }
 
@@ -932,14 +843,13 @@ struct Plan {
 //                          compiled in is refused here, with a message, and the default is used
 //   OMNI_MOE_TILE_WN       2: tile kernel of 256 x 128 instead of 256 x 256
 //   OMNI_MOE_TILE_LINES    0: the 256 x 256 tile kernel keeps the fragment layout of the activation operand
-//   OMNI_MOE_TILE_PAIR     0: every block of the tile kernel takes one tile (large launches: two)
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
 //   OMNI_MOE_EQUAL_PROGRESS bit 0: the stream kernel of GEMM1 lowers the issue priority of its wavefronts as they
 //                          advance (default 1), bit 1: that of GEMM2 too (measured slower in every geometry)
 struct Tuning {
-  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1, tile_pair = 1;
+  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
   bool have[3] = {false, false, false};
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
@@ -957,7 +867,6 @@ Tuning read_tuning() {
   r.rowq = geti("OMNI_MOE_ROWQ", 0);
   r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
   r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
-  r.tile_pair = geti("OMNI_MOE_TILE_PAIR", 1);
   for (int kind = 1; kind <= 2; ++kind) {
     const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
     const char* e = getenv(name);
@@ -1102,21 +1011,16 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, si
   const int wn = tile_wn(KIND, units);
   a.tile_gx = units / ((KIND == 1) ? 2 * wn : 4 * wn);
   a.tile_gy = (int)((M_cap + BM - 1) / BM + Gt);
-  // Two column tiles per block for the bulk of a large launch (line layout, at least 8 tiles per CU in the
-  // worst case): the column count of a patch is then even, so that a pair stays inside one row of its patch.
-  const int cus = device_cu_count();
-  a.tile_pair = wn == 4 && tile_lines(a.Kdim) && tuning().tile_pair && a.tile_gx % 2 == 0 && cus > 0 &&
-                (int64_t)a.tile_gy * a.tile_gx >= (int64_t)8 * cus;
   a.tile_pc = 1;
   for (int c = 1; c <= 8; ++c)
-    if (a.tile_gx % c == 0 && (!a.tile_pair || c % 2 == 0)) a.tile_pc = c;
-  a.tile_pr = 4;  // measured at 8192 tokens with 4 columns per patch: 8 rows per patch 2 % slower, 16 rows 5 %
+    if (a.tile_gx % c == 0) a.tile_pc = c;
   // one block per real tile (the kernel numbers them from the row counts in device memory; ids past
   // the real tiles leave at once) plus, when the last partial round is split, up to one round of helpers
   int64_t nblocks = (int64_t)a.tile_gy * a.tile_gx;
   a.tile_slots = 0;
   a.tail_cnt = nullptr;
   a.tail_part = nullptr;
+  const int cus = device_cu_count();
   if (tail_ws && tail_bytes >= TILE_TAIL_BYTES && cus > 0 && tuning().tile_tail) {
     const size_t slot_bytes = (size_t)2 * wn * 8 * 16 * WAVE * sizeof(int32_t);
     const int blocks_per_cu = (wn == 4) ? 1 : 2;

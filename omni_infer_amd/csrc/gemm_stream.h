@@ -24,8 +24,7 @@ struct GemmArgs {
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
   int32_t* acc_dbg;    // [M_cap, N], nullable
-  int tile_gx, tile_gy, tile_pc, tile_pr;  // tile kernel: column tiles, row blocks (worst case), columns and rows of a patch
-  int tile_pair;                  // tile kernel, line layout: blocks of the bulk take two neighbouring column tiles each
+  int tile_gx, tile_gy, tile_pc;  // tile kernel: column tiles, row blocks (worst case), columns of a patch
   int tile_slots;                 // tile kernel: blocks the chip runs at once
   int tile_split_max;             // tile kernel: most shares a tile of the last partial round is split into
   int32_t* tail_cnt;              // tile kernel: arrival counters of the split tiles (zero at launch), or null
