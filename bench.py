@@ -95,8 +95,14 @@ def make_inputs(cfg, dev):
         n = max(1, int(round(H * cfg["outlier"])))
         ch = torch.randperm(H, generator=g)[:n]
         x[:, ch] *= 50.0
-    logits = torch.full((T, E), -30.0)
-    logits[:, :n_local] = torch.randn(T, n_local, generator=g)
+    if cfg.get("routing") == "global_filter":
+        # every expert of the model can be chosen: what a rank sees after the all-gather of the tokens, of which
+        # it keeps the assignments to its own experts (about T rows)
+        logits = torch.randn(T, E, generator=g)
+    else:
+        # local_dense: every token's K experts are local ones (what a rank receives after a dispatch: K * T rows)
+        logits = torch.full((T, E), -30.0)
+        logits[:, :n_local] = torch.randn(T, n_local, generator=g)
     bias = torch.randn(E, generator=g) * 0.01
     return x.to(torch.bfloat16).to(dev), logits.to(dev), bias.to(dev)
 
@@ -339,6 +345,39 @@ def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_ste
     return res, step
 
 
+def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
+    """The prefill token count with the routing of the all-gather form of expert parallelism (router over all
+    256 experts, the local range filter keeps about T assignments): layer time against both rooflines."""
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+    cfg = dict(SHAPES["prefill"], routing="global_filter")
+    T, H, I, K, n_local = cfg["T"], cfg["H"], cfg["I"], cfg["K"], cfg["n_local"]
+    x, logits, bias = make_inputs(cfg, dev)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, 1, ops._DT[rows_dtype])
+    workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+
+    def step(i):
+        ws = sets[i % len(sets)]
+        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
+                                             cfg["scale"], 1e-20)
+        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
+                                  (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out,
+                                  rows_dtype=rows_dtype)
+
+    ms, _ = time_steps(step, steps, warmup)
+    w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
+    counts = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR).counts.cpu()
+    rows_routed, active = int(counts.sum()), int((counts > 0).sum()) + 1
+    M_cap = T * K + T
+    return {"routing": "router over all 256 experts, assignments to the 32 local ones kept", "tokens": T,
+            "rows_routed": rows_routed, "rows_of_busiest_expert": int(counts.max()), "active_groups": active,
+            "rows_dtype": str(rows_dtype).split(".")[-1], "layer_us": ms * 1e3, "steps": steps,
+            "gemm1_kernel": ops.gemm_kernel_name(1, T, K, n_local, T, M_cap, H, I),
+            "hbm_frac": algorithmic_bytes_layer(cfg, active) / (ms * 1e-3) / HBM_PEAK,
+            "int8_frac": algorithmic_ops_layer(cfg, rows_routed) / (ms * 1e-3) / INT8_PEAK}
+
+
 def measure_block(name, ws, steps, warmup, dev):
     """The whole MoE block through DeepseekMoE.forward (gate GEMM, router, layer; fused body): what a model
     pays per layer call.  Weights are those of one weight set (no rotation: about the cache-resident share
@@ -540,6 +579,7 @@ def main():
             alt, _ = measure_layer("prefill", sets, pre_steps, 3, other, True, dev, kernel_steps=pre_steps)
             pre["other_rows_dtype"] = {k: alt[k] for k in ("rows_dtype", "layer_us", "int8_frac")}
             pre["other_rows_dtype"]["gemm2_kernel_us"] = alt["roofline_gemm2"]["kernel_us"]
+            pre["global_filter"] = measure_global_filter(sets, max(20, pre_steps), 3, rows_dtype, dev)
 
     head = dec if dec is not None else pre
     result = {
@@ -558,7 +598,7 @@ def main():
     if dec is not None and pre is not None:
         result["prefill"] = {k: pre[k] for k in ("workload", "tokens", "rows_routed", "rows_dtype", "layer_us", "steps",
                                                  "algorithmic_ops", "int8_frac", "single_step_us", "roofline_gemm1",
-                                                 "roofline_gemm2", "other_rows_dtype")}
+                                                 "roofline_gemm2", "other_rows_dtype", "global_filter")}
         if "cpu_baseline" in pre:
             result["prefill"]["gpu_vs_oracle_rel_err"] = pre["cpu_baseline"]["gpu_vs_oracle_rel_err"]
             result["prefill"]["gpu_vs_oracle_bit_exact"] = pre["cpu_baseline"]["gpu_vs_oracle_bit_exact"]
