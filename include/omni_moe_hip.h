@@ -221,6 +221,35 @@ int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int
                               size_t buf_bytes);
 
 /*
+ * Expert placement (redundant copies of experts over the devices of an EP group).
+ *
+ * omni_placement_tables is HOST code on HOST pointers: from a placement pattern [world][layers][experts] of 0/1
+ * (1: that device deploys that expert in that layer) it writes
+ *   position_to_expert [layers][num_deploy] (may be NULL): device r owns the positions [r*P, (r+1)*P),
+ *       P = num_deploy / world, and its deployed experts take them in ascending expert id; unused positions
+ *       hold -1 (omni/accelerators/placement/omni_planner/cpp/placement_mapping.cpp:223-257);
+ *   selector [layers][experts]: the position that `rank` routes a logical expert to: its own copy, else one of
+ *       the copies on its host (devices_per_host devices per host), else one of the others, each set shared
+ *       out by rank modulo the size of the set, in ascending position order; an expert without any copy keeps 0
+ *       (placement_mapping.cpp:374-427).
+ * A pattern entry other than 0/1 or a device with more than P experts is rejected.
+ *
+ * omni_moe_remap_ids: out[i] = map[ids[i]] for 0 <= ids[i] < n_map, other ids are copied; `map` is one layer's
+ * row of the selector in device memory.  Replaces OmniPlanner.plan (omni_planner.py:244-274, the lookup at :273),
+ * called from FusedMoE.apply_expert_load_balance (omni/models/common/layers/moe/fused_moe/layer.py:273-286).
+ * out may be ids.
+ *
+ * omni_moe_record_activation: counts[e] = (counts[e] + tokens_per_expert[e]) mod modulus for the n deployed
+ * experts of the rank (int64 counters of one layer, int32 token counts as omni_moe_permute writes them).
+ * Replaces OmniPlanner.record_activation (omni_planner.py:337-343; called at fused_moe.py:652,746).
+ */
+int omni_placement_tables(const int32_t* pattern, int world, int layers, int experts, int rank,
+                          int devices_per_host, int num_deploy, int32_t* position_to_expert, int32_t* selector);
+int omni_moe_remap_ids(const int32_t* ids, int64_t n, const int32_t* map, int n_map, int32_t* out, void* stream);
+int omni_moe_record_activation(int64_t* counts, const int32_t* tokens_per_expert, int n, int64_t modulus,
+                               void* stream);
+
+/*
  * The OMNI_MOE_* tuning variables (kernel choice, tile shape, split tiles ...) are read from the environment
  * once, at the first GEMM call of the process.  This reads them again: for tests and tuning runs that change
  * them inside one process.  Not to be called while another thread launches GEMMs.  No counterpart in the

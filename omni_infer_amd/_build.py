@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libomni_moe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["route.hip", "quant.hip", "norm.hip", "permute.hip", "gemm.hip", "combine.hip", "diag.hip"]
+SOURCES = ["route.hip", "quant.hip", "norm.hip", "permute.hip", "gemm.hip", "combine.hip", "placement.hip", "diag.hip"]
 
 # -ffp-contract=off: every fp32 operation of the kernels rounds once (the parity contract).
 # The packed-fp32 feature is switched off for the device pass; the host pass does not know it

@@ -32,6 +32,9 @@ SIGNATURES = {
     "omni_moe_gemm2_dequant": (I, [P, P, P, P, P, P, I, P, I, I, I, c_int64, I, P, P, P, c_size_t, P]),
     "omni_moe_gemm2_workspace_bytes": (c_size_t, [I, I, c_int64, I, I]),
     "omni_moe_gemm_kernel_name": (I, [I, I, I, I, I, c_int64, I, I, P, c_size_t]),
+    "omni_placement_tables": (I, [P, I, I, I, I, I, I, P, P]),
+    "omni_moe_remap_ids": (I, [P, c_int64, P, I, P, P]),
+    "omni_moe_record_activation": (I, [P, P, I, c_int64, P]),
     "omni_moe_reload_tuning": (None, []),
     "omni_diag_mfma_i8_rate": (I, [P, c_size_t, I, I, P, P]),
     "omni_moe_combine": (I, [P, I, P, P, I, I, I, I, I, P, P, P, P, P]),
@@ -48,7 +51,7 @@ OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 
 OMNI_STATIC_SCRATCH_BYTES = 64 << 20
-ABI_VERSION = 4   # omni_moe_abi_version() of the header these signatures were written from
+ABI_VERSION = 5   # omni_moe_abi_version() of the header these signatures were written from
 
 _lib = None
 

@@ -32,6 +32,7 @@ class ModelOperatorOptConfig:
     gmm_nz: bool = False
     moe_dispatch_combine: bool = True
     use_omni_placement: bool = False
+    omni_placement_config_path: str = None
     enable_moe_expert_parallel: bool = True
     opt_w2_scale_cast: bool = False
     pd_seperate_prefill: bool = False

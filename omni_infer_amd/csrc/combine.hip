@@ -18,7 +18,7 @@ void omni_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 extern "C" const char* omni_moe_last_error(void) { return g_err; }
-extern "C" int omni_moe_abi_version(void) { return 4; }
+extern "C" int omni_moe_abi_version(void) { return 5; }
 
 namespace {
 

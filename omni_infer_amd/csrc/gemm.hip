@@ -264,7 +264,7 @@ struct LineCtx {
   int a_off[2][2];  // [k-step parity][half]: v4i index of the lane's A operand in a super-stage, row tile 0
   int b_off[2];     // same for the two 32-channel tiles of the wavefront, half 0
 };
-constexpr int LINE_LPS = 4;  // loads per k-step per wavefront: 2 A instructions (8 rows each), 2 B fragments
+[[maybe_unused]] constexpr int LINE_LPS = 4;  // loads per k-step per wavefront: 2 A instructions (8 rows each), 2 B fragments
 
 // the A loads of parity E fill rows [128 E, 128 E + 128) of a super-stage
 template <int E>

@@ -439,3 +439,55 @@ def moe_w8a8_layer_static(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk
                                             _ptr(out), _stream())
     L.check(rc, "omni_moe_w8a8_layer_static")
     return out
+
+
+# ----------------------------------------------------------------------------- expert placement
+def placement_tables(pattern: torch.Tensor, rank: int, devices_per_host: int, num_deploy: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Host tables of a placement pattern [world, layers, experts] (0/1, CPU): ``position_to_expert``
+    [layers, num_deploy] (-1: unused position) and ``selector`` [layers, experts], the position ``rank`` routes
+    each logical expert to (placement_mapping.cpp:223-257, :374-427).  Both are CPU int32 tensors."""
+    if pattern.is_cuda or pattern.dim() != 3:
+        raise ValueError("placement pattern must be a CPU tensor [world, layers, experts]")
+    pat = pattern.to(torch.int32).contiguous()
+    world, layers, experts = pat.shape
+    pos = torch.empty(layers, max(int(num_deploy), 0), dtype=torch.int32)
+    sel = torch.empty(layers, experts, dtype=torch.int32)
+    rc = L.lib().omni_placement_tables(pat.data_ptr(), world, layers, experts, int(rank), int(devices_per_host),
+                                       int(num_deploy), pos.data_ptr(), sel.data_ptr())
+    L.check(rc, "omni_placement_tables")
+    return pos, sel
+
+
+def remap_ids(ids: torch.Tensor, expert_map: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``embedding(ids, expert_map).squeeze(-1)`` of OmniPlanner.plan (omni_planner.py:273): every id becomes
+    ``expert_map[id]``; int32 in, int32 out (``out`` may be ``ids``)."""
+    _need_gpu(ids, expert_map)
+    if ids.dtype != torch.int32:
+        ids = ids.to(torch.int32)
+    ids = ids.contiguous()
+    expert_map = expert_map.reshape(-1)
+    if expert_map.dtype != torch.int32 or not expert_map.is_contiguous():
+        expert_map = expert_map.to(torch.int32).contiguous()
+    if out is None:
+        out = torch.empty_like(ids)
+    elif out.dtype != torch.int32 or not out.is_contiguous() or out.numel() != ids.numel():
+        raise ValueError("remap_ids: out must be a contiguous int32 tensor of the ids' size")
+    rc = L.lib().omni_moe_remap_ids(_ptr(ids), ids.numel(), _ptr(expert_map), expert_map.numel(), _ptr(out), _stream())
+    L.check(rc, "omni_moe_remap_ids")
+    return out
+
+
+def record_activation(counts: torch.Tensor, tokens_per_expert: torch.Tensor, modulus: int) -> torch.Tensor:
+    """``counts = (counts + tokens_per_expert) % modulus`` in place (omni_planner.py:337-343): int64 counters of
+    one layer, int32 token counts of the rank's deployed experts."""
+    _need_gpu(counts, tokens_per_expert)
+    if counts.dtype != torch.int64 or not counts.is_contiguous():
+        raise ValueError("record_activation: counts must be a contiguous int64 tensor (it is updated in place)")
+    n = counts.numel()
+    if tokens_per_expert.numel() != n:
+        raise ValueError("record_activation: one token count per counter")
+    if tokens_per_expert.dtype != torch.int32 or not tokens_per_expert.is_contiguous():
+        tokens_per_expert = tokens_per_expert.to(torch.int32).contiguous()
+    rc = L.lib().omni_moe_record_activation(_ptr(counts), _ptr(tokens_per_expert), n, int(modulus), _stream())
+    L.check(rc, "omni_moe_record_activation")
+    return counts

@@ -23,6 +23,7 @@ from torch import nn
 from .. import hip_ops as ops
 from ..config import model_extra_config
 from ..distributed import get_ep_group, get_world_group
+from ..placement import OmniPlanner
 from .activation import SiluAndMul
 from .layer import FusedMoE
 from .linear import MergedReplicatedLinear, ReplicatedLinear
@@ -72,7 +73,7 @@ class DeepseekMoE(nn.Module):
     norm_topk_prob, scoring_func, topk_method, routed_scaling_factor, hidden_act,
     first_k_dense_replace."""
 
-    def __init__(self, config, quant_config=None, prefix: str = "", device=None):
+    def __init__(self, config, quant_config=None, prefix: str = "", device=None, planner=None):
         super().__init__()
         self.prefix = prefix
         self.ep_size = get_ep_group().world_size
@@ -94,13 +95,24 @@ class DeepseekMoE(nn.Module):
         else:
             self.gate.e_score_correction_bias = None
         self.global_rank = get_world_group().rank_in_group
+        # deepseek_moe.py:161-176: with a placement the routed experts are addressed by deployed position
+        self.planner = self.moe_layer_idx = self.expert_mapping = None
+        if model_extra_config.operator_opt_config.use_omni_placement:
+            self.planner = planner if planner is not None else OmniPlanner(
+                config_file=model_extra_config.operator_opt_config.omni_placement_config_path, device=device or "cuda",
+                rank=get_world_group().rank_in_group, world_size=get_world_group().world_size,
+                num_experts=config.n_routed_experts, num_redundancy_shared_expert_rank=self.redundancy_shared_expert_num)
+            self.moe_layer_idx = OmniPlanner.get_deepseek_v3_moe_layer_idx(
+                f"{prefix}.experts", getattr(config, "first_k_dense_replace", 3))
+            self.expert_mapping = self.planner.expert_mapping_on_current_layer(self.moe_layer_idx)
         self.experts = FusedMoE(
             num_experts=config.n_routed_experts, top_k=config.num_experts_per_tok, hidden_size=config.hidden_size,
             intermediate_size=config.moe_intermediate_size, reduce_results=False, renormalize=config.norm_topk_prob,
             quant_config=quant_config, use_grouped_topk=True, num_expert_group=config.n_group,
             topk_group=config.topk_group, prefix=f"{prefix}.experts", scoring_func=config.scoring_func,
             e_score_correction_bias=self.gate.e_score_correction_bias,
-            first_k_dense_replace=getattr(config, "first_k_dense_replace", 3), device=device)
+            first_k_dense_replace=getattr(config, "first_k_dense_replace", 3), device=device,
+            planner=self.planner, moe_layer_idx=self.moe_layer_idx, expert_mapping=self.expert_mapping)
         self.shared_experts = None
         if config.n_shared_experts is not None:
             self.shared_experts = ReplicatedDeepseekMLP(
@@ -122,6 +134,13 @@ class DeepseekMoE(nn.Module):
             for lin in (self.shared_experts.gate_up_proj, self.shared_experts.down_proj):
                 if lin.quant_method is not None:
                     lin.quant_method.process_weights_after_loading(lin)
+
+    def _positions_per_rank(self) -> int:
+        """Width of a rank's range of expert ids: its experts, or with a placement the deployed positions every
+        rank is given (compressed_tensors_moe.py:126-128; fused_moe.py:510)."""
+        if self.planner is not None and self.planner.is_moe_layer(self.moe_layer_idx):
+            return self.planner.get_max_num_deployed_expert_per_rank()
+        return self.local_expert_num
 
     def _route(self, hidden_states, attn_metadata=None):
         """``self.gate.forward(hidden_states.float())`` + ``FusedMoE.select_experts`` (deepseek_moe.py:253-256,
@@ -181,7 +200,7 @@ class DeepseekMoE(nn.Module):
             hidden_states = hidden_states["x"]
         topk_weights, topk_ids = self._route(hidden_states, attn_metadata)
         e = self.experts
-        lo = self.global_rank * self.local_expert_num
+        lo = self.global_rank * self._positions_per_rank()
         shared = None
         if self.shared_experts is not None:
             gu, dn = self.shared_experts.gate_up_proj, self.shared_experts.down_proj

@@ -62,7 +62,13 @@ class FusedMoE(torch.nn.Module):
         self.quant_mode = DYNAMIC_QUANT_MODE
         if self.quant_method is None:
             raise RuntimeError("self.quant_method must not be None")
-        self.quant_method.create_weights(layer=self, num_experts=num_experts, hidden_size=hidden_size,
+        # layer.py:240-246: a rank that deploys redundant copies holds that many more experts
+        num_of_redundant_experts = 0
+        if model_extra_config.operator_opt_config.use_omni_placement and self.planner is not None:
+            num_of_redundant_experts = self.planner.get_num_of_redundant_experts(
+                moe_layer_idx=self.moe_layer_idx, num_expert_per_device_origin=num_experts,
+                rank_device=get_ep_group().rank_in_group - model_extra_config.parall_config.redundancy_shared_expert_num)
+        self.quant_method.create_weights(layer=self, num_experts=num_experts + num_of_redundant_experts, hidden_size=hidden_size,
                                          intermediate_size_per_partition=self.intermediate_size_per_partition,
                                          params_dtype=params_dtype, weight_loader=self.weight_loader,
                                          **({"device": kwargs["device"]} if "device" in kwargs else {}))
@@ -72,8 +78,8 @@ class FusedMoE(torch.nn.Module):
             raise ValueError("Only softmax scoring function is supported for non-grouped topk.")
 
     def apply_expert_load_balance(self, topk_ids: torch.Tensor, best_topk_ids: Optional[torch.Tensor] = None):
-        """layer.py:273-299: the placement planner's remap when a planner was given (none is built here), then the
-        forced balance of the ``best_ep`` flag: a prefill instance (``ROLE=prefill``) replaces the routing by
+        """layer.py:273-299: the placement planner's remap of the ids to deployed positions when a planner was
+        given, then the forced balance of the ``best_ep`` flag: a prefill instance (``ROLE=prefill``) replaces the routing by
         the ids 0..255 dealt round robin, eight per token (the reference hard-codes 256 experts and top-8 at
         :291-292); elsewhere the caller's ``best_topk_ids`` are taken when given."""
         if self.planner is not None:
@@ -178,9 +184,15 @@ class FusedMoE(torch.nn.Module):
 
     # ------------------------------------------------------------------ checkpoint loading
     def _local_expert(self, expert_id: int) -> int:
-        """Global -> local expert id, -1 if another rank owns it (layer.py:427-430)."""
+        """Global -> local expert id, -1 if another rank owns it (layer.py:414-430); with a placement the pattern
+        says whether the rank deploys the expert and at which local position (:417-424)."""
         if not model_extra_config.operator_opt_config.enable_moe_expert_parallel:
             return expert_id
+        if model_extra_config.operator_opt_config.use_omni_placement and self.planner is not None:
+            ep_rank = get_ep_group().rank_in_group - model_extra_config.parall_config.redundancy_shared_expert_num
+            exists_locally, local_pos = self.planner.is_expert_on_current_rank(self.moe_layer_idx, expert_id, ep_rank,
+                                                                               self.num_experts)
+            return local_pos if exists_locally else -1
         lo = get_ep_group().rank_in_group * self.num_experts
         return expert_id - lo if lo <= expert_id < lo + self.num_experts else -1
 

@@ -93,6 +93,10 @@ class AscendCompressedTensorsW8A8Int8MoEMethod:
         """compressed_tensors_moe.py:116-219, same branch conditions."""
         opt = model_extra_config.operator_opt_config
         n_local = self.n_routed_experts
+        max_num_deployed_expert_per_rank = n_local   # :126-128
+        planner = getattr(layer, "planner", None)
+        if opt.use_omni_placement and planner is not None and planner.is_moe_layer(layer.moe_layer_idx):
+            max_num_deployed_expert_per_rank = planner.get_max_num_deployed_expert_per_rank()
         if opt.enable_moe_expert_parallel:
             is_prefill = attn_metadata is None or attn_metadata.prefill is not None
             if opt.prefill_dispatch_combine or (opt.moe_dispatch_combine and not is_prefill):
@@ -107,7 +111,7 @@ class AscendCompressedTensorsW8A8Int8MoEMethod:
                     hidden_states=x, pertoken_scale=pertoken_scale, w1=layer.w13_weight, w2=layer.w2_weight,
                     w1_scale=layer.w13_weight_scale, w2_scale=layer.w2_weight_scale, topk_weights=topk_weights,
                     topk_ids=topk_ids, n_routed_experts=n_local, is_prefill=is_prefill,
-                    max_num_deployed_expert_per_rank=n_local)
+                    max_num_deployed_expert_per_rank=max_num_deployed_expert_per_rank)
             if self.warm_up:
                 self.warm_up = False
             return out
@@ -160,6 +164,9 @@ def fused_experts_w8a8_one_rank_dispatch_combine(layer, x: torch.Tensor, topk_we
     else:
         raise ValueError("dispatch/combine takes unquantised tokens")
     rows_q, rows_s = ops.moe_gather_rows(x_q, x_s, p)
+    planner = getattr(layer, "planner", None)
+    if model_extra_config.operator_opt_config.use_omni_placement and planner is not None:
+        planner.record_activation(layer.moe_layer_idx, p.counts, True)   # fused_moe.py:745-746
     rows = moe_expert_quant_farword(rows_q, layer.w13_weight, layer.w2_weight, layer.w13_weight_scale,
                                     layer.w2_weight_scale, p.counts, torch.bfloat16, 2, rows_s)
     return ops.moe_combine(rows, topk_weights, p.src_to_dst, L.OMNI_IDX_TOKEN_MAJOR, L.OMNI_ORDER_K)
