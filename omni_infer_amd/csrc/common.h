@@ -289,7 +289,7 @@ __device__ __forceinline__ bool row_blocks_find(const RowBlockScan& s, const int
   return true;
 }
 // The same row blocks numbered by weight: first the heavy blocks of all groups in group order (full blocks, and
-// last blocks with more than `light_max` rows), then the light last blocks of the groups that have one.  A
+// last blocks that are not light, see last_block_is_light), then the light last blocks of the groups that have one.  A
 // kernel whose blocks cost the same from light_max + 1 rows on can then deal out equal work first and keep the
 // cheap blocks for the end.
 struct RowBlockKinds {
@@ -299,8 +299,20 @@ struct RowBlockKinds {
   int total_h, total_l;
   bool small;
 };
-__device__ __forceinline__ int heavy_blocks(int c, int BM, int light_max) { return c / BM + ((c % BM) > light_max); }
-__device__ __forceinline__ int light_blocks(int c, int BM, int light_max) { return (c % BM) > 0 && (c % BM) <= light_max; }
+// A group's last block is light when it has at most light_max rows -- except in a group of exactly one full block
+// and a few rows more: there the small block stays next to the full one, whose weight panel it shares (deferred
+// to the end it would fetch that panel a second time, and with one full block per group that doubles the traffic).
+__device__ __forceinline__ bool last_block_is_light(int c, int BM, int light_max) {
+#ifdef OMNI_PROBE_LIGHT_ALWAYS
+  return (c % BM) > 0 && (c % BM) <= light_max;
+#else
+  return (c % BM) > 0 && (c % BM) <= light_max && c / BM != 1;
+#endif
+}
+__device__ __forceinline__ int heavy_blocks(int c, int BM, int light_max) {
+  return c / BM + ((c % BM) > 0 && !last_block_is_light(c, BM, light_max));
+}
+__device__ __forceinline__ int light_blocks(int c, int BM, int light_max) { return last_block_is_light(c, BM, light_max); }
 __device__ __forceinline__ RowBlockKinds row_block_kinds_scan(const int32_t* __restrict__ offsets, int G, int extra_rows,
                                                               int BM, int light_max) {
   const int lane = threadIdx.x & (WAVE - 1);
