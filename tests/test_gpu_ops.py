@@ -461,3 +461,31 @@ def test_layer_entry_tile_sweep(ops, tuning, T, K, n_local, E, H, I, shared, see
     out = ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), lo, lo + n_local, d["w13"], d["s13"], d["w2"], d["s2"],
                              sh, H=H, I=I)
     _eq(out, want, f"layer output T={T} K={K} n_local={n_local}/{E} H={H} I={I} shared={shared}")
+
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_tile_numbering_row_count_edges(ops, tuning, shared):
+    """Groups whose row counts sit on every edge of the tile numbering: empty, one row, 96 and 97 rows (light /
+    heavy last block), one full block, one full block plus a few rows (the small block that stays next to its
+    full one), plus 96 and 97, two and more full blocks with and without a light tail."""
+    tuning(OMNI_MOE_FORCE_KERNEL=2)
+    counts = [0, 1, 96, 97, 256, 257, 300, 352, 353, 512, 513, 608, 609, 0, 768 + 40, 255]
+    n_local, H, I = len(counts), 256, 128
+    E = n_local + 3
+    T = sum(counts) + 50                              # 50 tokens go to experts of other ranks
+    g = gen(4242)
+    ids = torch.cat([torch.full((c,), e + 2, dtype=torch.int32) for e, c in enumerate(counts)] +
+                    [torch.full((25,), 0, dtype=torch.int32), torch.full((25,), E - 1, dtype=torch.int32)])
+    ids = ids[torch.randperm(T, generator=g)].view(T, 1)
+    w = torch.rand(T, 1, generator=g)
+    lay = Layer(n_local, H, I, seed=4242, shared=shared)
+    x = tokens(T, H, 4243)
+    xq, xs = O.dynamic_quant(x)
+    want = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (2, 2 + n_local))
+    if shared:
+        want = (want.float() + O.shared_expert_mlp(x, *lay.shared).float()).to(torch.bfloat16)
+    d = lay.to_device()
+    sh = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]) if shared else None
+    out = ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), 2, 2 + n_local, d["w13"], d["s13"], d["w2"], d["s2"],
+                             sh, H=H, I=I)
+    _eq(out, want, f"row-count edges shared={shared}")
