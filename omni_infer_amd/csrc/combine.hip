@@ -255,13 +255,19 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
   int32_t* src_to_dst = (int32_t*)(ws + L.src_to_dst);
   int32_t* offsets = (int32_t*)(ws + L.offsets);
   bool sorted = false;
+  const int extra = with_shared ? T : 0;
+  // When both grouped GEMMs run the tile kernel, the arrival counters of their split tiles are cleared by the
+  // sorting kernel below (the first kernel to run that has a single-block part), not by two launches of their own.
+  int cnt_words = 0;
+  size_t tail_bytes = 0;
+  void* const tail = omni_tile_tail_area(T, K, G, extra, L.M_cap, H, I, ws + L.g1_ws, L.g1_bytes, &cnt_words, &tail_bytes);
   if (x_dtype != -1) {
     // the quantisation and the sort do not depend on each other: one launch when both are small
     rc = 1;
     if (x_dtype == OMNI_DT_BF16)
       rc = omni_quant_permute_fused(x, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), topk_ids, K, lo, hi,
                                     OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts), offsets,
-                                    stream);
+                                    (int32_t*)tail, cnt_words, stream);
     if (rc < 0) return rc;
     sorted = rc == 0;
     if (!sorted) {
@@ -272,19 +278,20 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
     xs = (const float*)(ws + L.x_s);
   }
   if (!sorted) {
-    rc = omni_moe_permute(topk_ids, T, K, lo, hi, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts),
-                          offsets, ws + L.perm_ws, L.perm_bytes, stream);
+    rc = omni_moe_permute_clearing(topk_ids, T, K, lo, hi, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst,
+                                   (int32_t*)(ws + L.counts), offsets, ws + L.perm_ws, L.perm_bytes, (int32_t*)tail,
+                                   cnt_words, stream);
     if (rc) return rc;
   }
-  const int extra = with_shared ? T : 0;
-  rc = omni_moe_gemm1_swiglu_quant(xq, xs, sorted_src, OMNI_IDX_TOKEN_MAJOR, T, K, w13_packed, w13_scale, sh13_packed,
-                                   sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),
-                                   (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, stream);
+  rc = omni_gemm1_swiglu_quant_impl(xq, xs, sorted_src, OMNI_IDX_TOKEN_MAJOR, T, K, w13_packed, w13_scale, sh13_packed,
+                                    sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),
+                                    (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, tail != nullptr, stream);
   if (rc) return rc;
-  // GEMM1's scratch is free again once its row quantiser has run: GEMM2 takes it over
-  rc = omni_moe_gemm2_dequant((const int8_t*)(ws + L.h_q), (const float*)(ws + L.h_s), w2_packed, w2_scale, sh2_packed,
-                              sh2_scale, extra, offsets, G, H, I, L.M_cap, L.rows_dtype, ws + L.rows, nullptr,
-                              ws + L.g1_ws, L.g1_bytes, stream);
+  // GEMM1's scratch is free again once its row quantiser has run: GEMM2 takes it over (with cleared counters: the
+  // split-tile scratch of GEMM1, whose counter words for GEMM2 nobody has touched since the sorting kernel)
+  rc = omni_gemm2_dequant_impl((const int8_t*)(ws + L.h_q), (const float*)(ws + L.h_s), w2_packed, w2_scale, sh2_packed,
+                               sh2_scale, extra, offsets, G, H, I, L.M_cap, L.rows_dtype, ws + L.rows, nullptr,
+                               tail ? tail : (void*)(ws + L.g1_ws), tail ? tail_bytes : L.g1_bytes, tail != nullptr, stream);
   if (rc) return rc;
   return omni_moe_combine(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
                           nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,
@@ -337,8 +344,9 @@ extern "C" int omni_moe_w8a8_layer_static(const void* x, int x_dtype, const floa
   void* ptr = nullptr;
   const int rc = static_scratch_ptr(&ptr);
   if (rc) return rc;
-  // nothing in the scratch has to start at zero except the arrival counters of split tiles, and the tile
-  // launch clears those itself with a fill kernel; everything else is written before it is read
+  // nothing in the scratch has to start at zero except the arrival counters of split tiles, and those are cleared
+  // by a kernel of the call itself (the sorting kernel, or a fill kernel in front of the tile launch); everything
+  // else is written before it is read
   return omni_moe_w8a8_layer(x, x_dtype, x_scale_in, topk_w, topk_ids, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
                              w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, ptr,
                              (size_t)OMNI_STATIC_SCRATCH_BYTES, stream);

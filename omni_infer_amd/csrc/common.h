@@ -31,10 +31,30 @@ void omni_set_error(const char* fmt, ...);
     if (e__ != hipSuccess) OMNI_FAIL(OMNI_E_LAUNCH, "%s: %s", what, hipGetErrorString(e__)); \
   } while (0)
 
-// library-internal: bf16 row quantisation and assignment sort in one launch (permute.hip); 1 = not applicable
+// library-internal: bf16 row quantisation and assignment sort in one launch (permute.hip); 1 = not applicable.
+// zero_words (may be null) are cleared by the sorting block: the whole-layer entry has the arrival counters of
+// the later tile launches cleared here instead of by a launch of their own.
 int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float* scale, const int32_t* topk_ids, int K,
                              int lo, int hi, int idx_mode, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
-                             int32_t* offsets, void* stream);
+                             int32_t* offsets, int32_t* zero_words, int zero_n, void* stream);
+// library-internal: omni_moe_permute that also clears zero_words (in its single-block kernel)
+int omni_moe_permute_clearing(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode, int32_t* sorted_src,
+                              int32_t* src_to_dst, int32_t* counts, int32_t* offsets, void* workspace, size_t ws_bytes,
+                              int32_t* zero_words, int zero_n, void* stream);
+// library-internal (gemm.hip): the scratch of split tiles inside a GEMM1 workspace when both grouped GEMMs of a layer
+// call of this shape run the tile kernel (else null), with the number of counter words at its start that must be
+// zero before the first of the two launches; and the two GEMM entries with the promise that they are.
+void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, void* gemm1_ws,
+                          size_t gemm1_ws_bytes, int* counter_words, size_t* tail_bytes);
+int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode, int T,
+                                 int K, const int8_t* w13_packed, const float* w13_scale, const int8_t* w13_extra,
+                                 const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G, int H, int I,
+                                 int64_t M_cap, int flags, int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
+                                 size_t ws_bytes, bool counters_clean, void* stream);
+int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
+                            const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows, const int32_t* offsets,
+                            int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out, int32_t* acc_dbg,
+                            void* workspace, size_t ws_bytes, bool counters_clean, void* stream);
 
 // ---------------------------------------------------------------- specified transcendental
 // exp with a fixed operation sequence: clamp to [-87, 87], Cody-Waite reduction by ln2 split in

@@ -982,7 +982,9 @@ int tile_wn(int kind, int units) {
 // Scratch of the split tiles of a launch: arrival counters, then one slot of partial accumulators per
 // share.  At most `tile_slots` shares exist (splits x split tiles <= slots), a slot is the 256 x 64*WN
 // int32 tile of a block, and the slot count is capped so that the area has one size for every shape.
-constexpr size_t TILE_TAIL_CNT_BYTES = 4096;
+// (the counters of GEMM1 and of GEMM2 are different words, so that one clearing in front of both launches serves)
+constexpr int TILE_TAIL_CNT_WORDS = 1024;                                  // per kind of GEMM
+constexpr size_t TILE_TAIL_CNT_BYTES = 2 * TILE_TAIL_CNT_WORDS * sizeof(int32_t);
 constexpr size_t TILE_TAIL_PART_BYTES = (size_t)64 << 20;
 constexpr size_t TILE_TAIL_BYTES = TILE_TAIL_CNT_BYTES + TILE_TAIL_PART_BYTES;
 
@@ -1004,7 +1006,8 @@ int device_cu_count() {
 }
 
 template <int KIND>
-void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, size_t tail_bytes, hipStream_t st) {
+void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, size_t tail_bytes, bool counters_clean,
+                 hipStream_t st) {
   const int BM = 256;
   GemmArgs a = a0;
   const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
@@ -1026,12 +1029,12 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, si
     const int blocks_per_cu = (wn == 4) ? 1 : 2;
     int slots = cus * blocks_per_cu;
     if ((size_t)slots * slot_bytes > TILE_TAIL_PART_BYTES) slots = (int)(TILE_TAIL_PART_BYTES / slot_bytes);
-    if ((size_t)slots * sizeof(int32_t) > TILE_TAIL_CNT_BYTES) slots = (int)(TILE_TAIL_CNT_BYTES / sizeof(int32_t));
+    if (slots > TILE_TAIL_CNT_WORDS) slots = TILE_TAIL_CNT_WORDS;
     a.tile_slots = slots;
     a.tile_split_max = tuning().tile_split;
-    a.tail_cnt = (int32_t*)tail_ws;
+    a.tail_cnt = (int32_t*)tail_ws + (KIND - 1) * TILE_TAIL_CNT_WORDS;
     a.tail_part = (int32_t*)((char*)tail_ws + TILE_TAIL_CNT_BYTES);
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, st, a.tail_cnt, slots);
+    if (!counters_clean) hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, st, a.tail_cnt, slots);
     nblocks += slots;
   }
   dim3 grid((unsigned)nblocks), block(128 * wn);
@@ -1049,11 +1052,11 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, si
 }
 
 template <int KIND>
-int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, void* tail_ws, size_t tail_bytes, hipStream_t st,
-                  const char* what) {
+int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, void* tail_ws, size_t tail_bytes, bool counters_clean,
+                  hipStream_t st, const char* what) {
   const int units = (KIND == 1) ? a.N / 32 : a.N / 16;
   if (p.tile) {
-    launch_tile<KIND>(a, M_cap, units, tail_ws, tail_bytes, st);
+    launch_tile<KIND>(a, M_cap, units, tail_ws, tail_bytes, counters_clean, st);
   } else {
     const int mt = p.mt, nt = p.nt, d = p.d;
     if (units % (4 * nt) != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: %d output strips not divisible by %d", what, units, 4 * nt);
@@ -1113,6 +1116,29 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
                                            const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G,
                                            int H, int I, int64_t M_cap, int flags, int8_t* h_q, float* h_scale,
                                            int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream) {
+  return omni_gemm1_swiglu_quant_impl(x_q, x_scale, sorted_src, idx_mode, T, K, w13_packed, w13_scale, w13_extra,
+                                      w13_extra_scale, extra_rows, offsets, G, H, I, M_cap, flags, h_q, h_scale, acc_dbg,
+                                      workspace, ws_bytes, false, stream);
+}
+
+void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, void* gemm1_ws,
+                          size_t gemm1_ws_bytes, int* counter_words, size_t* tail_bytes) {
+  if (T <= 0 || K <= 0 || G < 0 || M_cap <= 0 || !gemm1_ws) return nullptr;
+  const Plan p1 = make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap);
+  const Plan p2 = make_plan<2>((int)M_cap, 1, G, extra_rows, I, H, M_cap);
+  if (!p1.tile || !p2.tile) return nullptr;
+  const size_t at = align256((size_t)M_cap * I * sizeof(float) + 256);
+  if (gemm1_ws_bytes < at + TILE_TAIL_BYTES) return nullptr;
+  *counter_words = 2 * TILE_TAIL_CNT_WORDS;
+  *tail_bytes = TILE_TAIL_BYTES;
+  return (char*)gemm1_ws + at;
+}
+
+int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode, int T,
+                                 int K, const int8_t* w13_packed, const float* w13_scale, const int8_t* w13_extra,
+                                 const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G, int H, int I,
+                                 int64_t M_cap, int flags, int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
+                                 size_t ws_bytes, bool counters_clean, void* stream) {
   int rc = check_group_args("gemm1", offsets, G, H, I, M_cap, extra_rows, w13_extra, w13_extra_scale);
   if (rc) return rc;
   if (M_cap == 0) return OMNI_OK;
@@ -1134,7 +1160,7 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
     float* y = (float*)workspace;
     a.y = y;
     void* tail_ws = (char*)workspace + align256((size_t)M_cap * I * sizeof(float) + 256);
-    rc = dispatch_gemm<1>(a, p, M_cap, tail_ws, TILE_TAIL_BYTES, st, "gemm1");
+    rc = dispatch_gemm<1>(a, p, M_cap, tail_ws, TILE_TAIL_BYTES, counters_clean, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
     launch_quant_rows_y(y, offsets, G, extra_rows, I, M_cap, h_q, h_scale, st);
@@ -1145,7 +1171,7 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
     // one k share: the stream kernel finishes y = silu(gate)*up itself (the workspace holds it, half
     // the bytes of the raw sums), then the row quantiser of the tile path
     a.y = (float*)workspace;
-    rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, st, "gemm1");
+    rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, false, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
     launch_quant_rows_y(a.y, offsets, G, extra_rows, I, M_cap, h_q, h_scale, st);
@@ -1155,7 +1181,7 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
   // split-k stream kernel: raw int32 partial sums, then one row kernel does the whole epilogue
   if (I > 256 * 16) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gemm1: intermediate size %d > 4096 in the small-batch path", I);
   a.part = (int32_t*)workspace;
-  rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, st, "gemm1");
+  rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, false, st, "gemm1");
   if (rc) return rc;
   if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;
   // few rows (decode): more threads per row shorten the per-thread chain of exp / divide sequences
@@ -1173,6 +1199,14 @@ extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, c
                                       int extra_rows, const int32_t* offsets, int G, int H, int I, int64_t M_cap,
                                       int out_dtype, void* rows_out, int32_t* acc_dbg, void* workspace, size_t ws_bytes,
                                       void* stream) {
+  return omni_gemm2_dequant_impl(h_q, h_scale, w2_packed, w2_scale, w2_extra, w2_extra_scale, extra_rows, offsets, G, H, I,
+                                 M_cap, out_dtype, rows_out, acc_dbg, workspace, ws_bytes, false, stream);
+}
+
+int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
+                            const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows, const int32_t* offsets,
+                            int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out, int32_t* acc_dbg,
+                            void* workspace, size_t ws_bytes, bool counters_clean, void* stream) {
   int rc = check_group_args("gemm2", offsets, G, H, I, M_cap, extra_rows, w2_extra, w2_extra_scale);
   if (rc) return rc;
   if (M_cap == 0) return OMNI_OK;
@@ -1188,7 +1222,7 @@ extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, c
   a.rows_out = rows_out; a.out_dtype = out_dtype; a.acc_dbg = acc_dbg; a.S = 1; a.M_cap = M_cap;
   Plan p = make_plan<2>(a.T, a.K, G, extra_rows, I, H, M_cap);
   if (workspace && ((uintptr_t)workspace % 256)) OMNI_FAIL(OMNI_E_INVALID, "gemm2: workspace must be 256-byte aligned");
-  return dispatch_gemm<2>(a, p, M_cap, workspace, workspace ? ws_bytes : 0, (hipStream_t)stream, "gemm2");
+  return dispatch_gemm<2>(a, p, M_cap, workspace, workspace ? ws_bytes : 0, counters_clean, (hipStream_t)stream, "gemm2");
 }
 
 extern "C" size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int H, int I) {

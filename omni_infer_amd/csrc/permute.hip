@@ -27,7 +27,13 @@ struct PermArgs {
   int32_t* offsets;
   int32_t* blk_hist;  // [nblk][NB] counts, then (after the scan) exclusive block bases
   int nblk;
+  int32_t* zero_words;  // cleared by the single-block kernel of the call (null: nothing to clear)
+  int zero_n;
 };
+
+__device__ __forceinline__ void clear_words(const PermArgs& a) {
+  for (int i = threadIdx.x; i < a.zero_n; i += 256) a.zero_words[i] = 0;
+}
 
 __device__ __forceinline__ int bucket_of(int id, int lo, int G) {
   int e = id - lo;
@@ -117,6 +123,7 @@ __device__ __forceinline__ void permute_single_body(const PermArgs& a) {
   __shared__ int tot[NB];
   __shared__ int off[NB + 1];
   const int passes = (a.n + 255) / 256;
+  clear_words(a);
   rank_chunk(a, 0, a.n, passes, whist, lrank);
   const int nb = a.G + 1;
   for (int b = threadIdx.x; b < nb; b += 256) tot[b] = whist[0][b] + whist[1][b] + whist[2][b] + whist[3][b];
@@ -159,6 +166,7 @@ __global__ __launch_bounds__(256) void permute_scan(PermArgs a) {
   __shared__ int tot[NB];
   __shared__ int off[NB + 1];
   const int nb = a.G + 1;
+  clear_words(a);
   for (int b = threadIdx.x; b < nb; b += 256) {
     int run = 0;
     // eight blocks' counts are requested together before their prefixes are written back
@@ -239,6 +247,13 @@ extern "C" size_t omni_moe_permute_workspace_bytes(int T, int K, int n_local) {
 extern "C" int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode,
                                 int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts, int32_t* offsets,
                                 void* workspace, size_t ws_bytes, void* stream) {
+  return omni_moe_permute_clearing(topk_ids, T, K, lo, hi, idx_mode, sorted_src, src_to_dst, counts, offsets, workspace,
+                                   ws_bytes, nullptr, 0, stream);
+}
+
+int omni_moe_permute_clearing(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode, int32_t* sorted_src,
+                              int32_t* src_to_dst, int32_t* counts, int32_t* offsets, void* workspace, size_t ws_bytes,
+                              int32_t* zero_words, int zero_n, void* stream) {
   if (T < 0 || K <= 0 || hi <= lo) OMNI_FAIL(OMNI_E_INVALID, "permute: bad sizes T=%d K=%d range=[%d,%d)", T, K, lo, hi);
   const int G = hi - lo;
   if (G > GMAX) OMNI_FAIL(OMNI_E_UNSUPPORTED, "permute: %d local experts > %d", G, GMAX);
@@ -249,7 +264,8 @@ extern "C" int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, i
   const int n = T * K;
   if (ws_bytes < omni_moe_permute_workspace_bytes(T, K, G)) OMNI_FAIL(OMNI_E_WORKSPACE, "permute: workspace %zu < %zu", ws_bytes, omni_moe_permute_workspace_bytes(T, K, G));
   hipStream_t st = (hipStream_t)stream;
-  PermArgs a{topk_ids, n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, (int32_t*)workspace, 0};
+  PermArgs a{topk_ids, n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, (int32_t*)workspace, 0,
+             zero_words, zero_words ? zero_n : 0};
   if (n <= CH_SINGLE) {
     hipLaunchKernelGGL(permute_single, dim3(1), dim3(256), 0, st, a);
     OMNI_CHECK_LAUNCH("permute_single");
@@ -268,12 +284,13 @@ extern "C" int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, i
 // assignments in one launch.  Returns 1 without launching when the shapes do not fit that kernel.
 int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float* scale, const int32_t* topk_ids, int K,
                              int lo, int hi, int idx_mode, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
-                             int32_t* offsets, void* stream) {
+                             int32_t* offsets, int32_t* zero_words, int zero_n, void* stream) {
   const int G = hi - lo;
   const int64_t n = (int64_t)T * K;
   if (T <= 0 || n > CH_SINGLE || G > GMAX || H % 8 != 0 || H > 8 * 256 * 4) return 1;
   if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((size_t)H * 2) % 16 != 0) return 1;
-  PermArgs a{topk_ids, (int)n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, nullptr, 0};
+  PermArgs a{topk_ids, (int)n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, nullptr, 0,
+             zero_words, zero_words ? zero_n : 0};
   dim3 grid((unsigned)T + 1), block(256);
   hipStream_t st = (hipStream_t)stream;
   if (H <= 8 * 256 * 1) hipLaunchKernelGGL(quant_permute_small<1>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
