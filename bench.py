@@ -428,7 +428,7 @@ def measure_block(name, ws, steps, warmup, dev):
 def bench_calib(args):
     """What the hardware delivers on this box, to read the layer's figures against (one JSON line):
     the int8 matrix instruction alone on zero and on random operands, the vendor library's plain int8 GEMM
-    (torch._int_mm) at the shapes of the two prefill GEMMs, and a device-to-device copy."""
+    (torch._int_mm) at the shapes of the two prefill GEMMs, a device-to-device copy and a kernel that only reads."""
     from omni_infer_amd import _lib as L
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -516,6 +516,17 @@ def bench_calib(args):
     dst = torch.empty_like(src)
     ms = ev_ms(lambda: dst.copy_(src), 10)
     res["copy_1GiB_read_plus_write_TBps"] = 2 * (1 << 30) / (ms * 1e-3) / 1e12
+    # a kernel that only reads (the library's diagnostic): the ceiling of the weight-streaming GEMMs of the decode step
+    del dst
+    best = (0.0, 0)
+    for per_cu in (4, 8, 16, 32, 64):
+        def rd():
+            L.check(lib.omni_diag_hbm_read_rate(src.data_ptr(), src.numel(), cus * per_cu, sink.data_ptr(), st),
+                    "omni_diag_hbm_read_rate")
+        tbps = (1 << 30) / (ev_ms(rd, 10) * 1e-3) / 1e12
+        res[f"read_1GiB_{per_cu}_blocks_per_cu_TBps"] = tbps
+        best = max(best, (tbps, per_cu))
+    res["read_1GiB_best_TBps"] = best[0]
     res["value"] = res["mfma_i8_gaussian_sigma30_pops"]
     print(json.dumps(res))
 

@@ -265,6 +265,13 @@ void omni_moe_reload_tuning(void);
  */
 int omni_diag_mfma_i8_rate(const int8_t* operands, size_t operand_bytes, int iters, int blocks, int32_t* sink,
                            void* stream);
+/*
+ * Diagnostic (no counterpart in the reference): `blocks` blocks of 256 threads read `bytes` of `buf` once, 16
+ * bytes per lane and request, eight requests of a lane in flight, and do nothing else.  The caller times the
+ * launch: bytes / time is what the memory system delivers to a kernel that only streams, the practical ceiling
+ * of the weight-streaming GEMMs.
+ */
+int omni_diag_hbm_read_rate(const void* buf, size_t bytes, int blocks, int32_t* sink, void* stream);
 
 /*
  * Weighted un-permute.  Replaces the routing half of npu_grouped_matmul_finalize_routing
