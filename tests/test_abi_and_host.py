@@ -74,6 +74,14 @@ def test_argument_validation_returns_codes(lib):
     assert lib.omni_moe_w8a8_layer(p, 0, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, 2, p,
                                    p, 1 << 30, None) == -1                                              # rows_dtype f16
     assert lib.omni_moe_w8a8_layer_workspace_bytes(4, 8, 32, 7168, 2048, 1, 2) == 0
+    assert lib.omni_moe_remap_ids(p, -1, p, 32, p, None) == -1
+    assert lib.omni_moe_remap_ids(p, 8, None, 32, p, None) == -1
+    assert lib.omni_moe_remap_ids(None, 0, None, 32, None, None) == 0                                    # nothing to do
+    assert lib.omni_moe_record_activation(p, p, 4, 0, None) == -1                                        # modulus
+    assert lib.omni_moe_record_activation(None, p, 4, 10, None) == -1
+    assert lib.omni_moe_record_activation(None, None, 0, 10, None) == 0
+    assert lib.omni_placement_tables(None, 1, 1, 1, 0, 1, 1, None, p) == -1
+    assert lib.omni_diag_hbm_read_rate(None, 1 << 20, 256, p, None) == -1
 
 
 def test_workspace_sizes(lib):
