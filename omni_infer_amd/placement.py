@@ -32,13 +32,20 @@ def _read_config(config_file: Optional[str]) -> dict:
         return {}
 
 
+def _device(device) -> torch.device:
+    """The reference's call sites say device="npu"; on this build that is the GPU."""
+    if isinstance(device, str) and device.startswith("npu"):
+        device = "cuda" + device[3:]
+    return torch.device(device)
+
+
 class ExpertMapping:
     """expert_mapping.py:12-281 for a static pattern.  ``pattern`` is [world, layers, experts] of 0/1 (an array,
     the path of a .npy file, or None for the base pattern: expert e on device e // (experts // world))."""
 
     def __init__(self, pattern=None, device="cuda", rank: int = 0, world_size: int = 1, num_devices_per_host: int = 8,
                  num_experts: int = 256, max_moe_layer_num: int = 58, max_redundant_per_rank: Optional[int] = None):
-        self.device = torch.device(device)
+        self.device = _device(device)
         self.rank = rank
         self.world_size = world_size
         self.num_devices_per_host = num_devices_per_host
@@ -156,7 +163,7 @@ class OmniPlanner:
         self.max_moe_layer_num = cfg.get("max_moe_layer_num", max_moe_layer_num)
         if self.max_moe_layer_num is None:
             raise ValueError("[Placement-Error]-max_moe_layer_num is not defined")
-        self.device = torch.device(device)
+        self.device = _device(device)
         # omni_planner.py:127-155: ranks that only hold redundant shared experts are not part of the expert pattern
         self.rank = rank - num_redundancy_shared_expert_rank
         self.world_size = world_size - num_redundancy_shared_expert_rank
