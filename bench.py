@@ -366,6 +366,17 @@ def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
                                   rows_dtype=rows_dtype)
 
     ms, _ = time_steps(step, steps, warmup)
+
+    def step_routed_only(i):
+        # the reference runs the shared expert on the rank's own tokens before the all-gather (deepseek_moe.py:244):
+        # on the gathered tokens only the routed experts are computed
+        ws = sets[i % len(sets)]
+        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
+                                             cfg["scale"], 1e-20)
+        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2, None, H=H, I=I,
+                                  workspace=workspace, out=out, rows_dtype=rows_dtype)
+
+    ms_routed, _ = time_steps(step_routed_only, steps, warmup)
     w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
     counts = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR).counts.cpu()
     rows_routed, active = int(counts.sum()), int((counts > 0).sum()) + 1
@@ -373,6 +384,9 @@ def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
     return {"routing": "router over all 256 experts, assignments to the 32 local ones kept", "tokens": T,
             "rows_routed": rows_routed, "rows_of_busiest_expert": int(counts.max()), "active_groups": active,
             "rows_dtype": str(rows_dtype).split(".")[-1], "layer_us": ms * 1e3, "steps": steps,
+            "routed_experts_only_us": ms_routed * 1e3,
+            "routed_experts_only_hbm_frac": algorithmic_bytes_layer(cfg, active - 1) / (ms_routed * 1e-3) / HBM_PEAK,
+            "routed_experts_only_int8_frac": 2 * rows_routed * (H * 2 * I + I * H) / (ms_routed * 1e-3) / INT8_PEAK,
             "gemm1_kernel": ops.gemm_kernel_name(1, T, K, n_local, T, M_cap, H, I),
             "hbm_frac": algorithmic_bytes_layer(cfg, active) / (ms * 1e-3) / HBM_PEAK,
             "int8_frac": algorithmic_ops_layer(cfg, rows_routed) / (ms * 1e-3) / INT8_PEAK}
