@@ -263,6 +263,9 @@ struct LineCtx {
   int w, lane;
   int a_off[2][2];  // [k-step parity][half]: v4i index of the lane's A operand in a super-stage, row tile 0
   int b_off[2];     // same for the two 32-channel tiles of the wavefront, half 0
+  // the 16x16x64 form: [k-step parity][upper 16 rows of the 32-row tile] and the four strips of the wavefront
+  int a16_off[2][2];
+  int b16_off[4];
 };
 [[maybe_unused]] constexpr int LINE_LPS = 4;  // loads per k-step per wavefront: 2 A instructions (8 rows each), 2 B fragments
 
@@ -390,6 +393,168 @@ __device__ __forceinline__ void line_k_loop(const LineCtx& c, int nk64, v4i* __r
       line_step<MTC, 1>(c, last, last_ss, sa1, sb0, sa0, sa2, sb1, X, Y, acc);
     }
   }
+#endif
+}
+
+// =====================================================================================
+// The same loop on v_mfma_i32_16x16x64_i8.  The chip lowers its clock with the switching activity of the matrix
+// datapath, and an instruction that folds 64 products into each of 256 accumulators switches less per product than
+// one that folds 32 into each of 1024: on the operand pattern of this kernel the 16x16x64 form sustains 4.1-4.3
+// POPS where the 32x32x32 form sustains 3.1-3.2.  The wavefront's piece, its 128 accumulator registers and the
+// bytes it reads from LDS are the same.  An instruction takes a whole k-step of 16 rows and 16 channels, so a
+// half step is now the lower or the upper 16 rows of every 32-row tile against all four strips of the wavefront:
+// the A operands of the two halves alternate between X and Y as before, the four B operands serve both halves
+// and are replaced one by one, each after the last instruction of the k-step that uses it.
+// Accumulators: acc[mt][t] (16 registers) holds four 16 x 16 results: registers 8 h + 4 s + i belong to rows
+// 16 h + 4 (lane / 16) + i of the tile and channel 16 s + lane % 16 of the pair of strips t.
+// =====================================================================================
+template <int MTC>
+struct Line16A { v4i a[MTC > 0 ? MTC : 1]; };
+
+template <int MTC, int E, int H>
+__device__ __forceinline__ void line16_read_a(const LineCtx& c, const v4i* __restrict__ src_a, Line16A<MTC>& o) {
+#pragma unroll
+  for (int mt = 0; mt < MTC; ++mt) o.a[mt] = src_a[c.a16_off[E][H] + mt * 256];
+}
+
+// the instructions of half H that use strip N of the wavefront
+template <int MTC, int H, int N>
+__device__ __forceinline__ void line16_mfma_n(const Line16A<MTC>& o, const v4i (&b)[4], v4i (&acc)[4][2][4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int mt = 0; mt < MTC; ++mt)
+    acc[mt][N >> 1][2 * H + (N & 1)] = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.a[mt], b[N], acc[mt][N >> 1][2 * H + (N & 1)], 0, 0, 0);
+#endif
+}
+
+// after the first MFMA: every LDS read, then every load, followed by one MFMA each while there are MFMAs left
+template <int D, int M, int V>
+__device__ __forceinline__ void line16_pin() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if constexpr (D > 0) {
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    if constexpr (M > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line16_pin<D - 1, (M > 0 ? M - 1 : 0), V>();
+  } else if constexpr (V > 0) {
+    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    if constexpr (M > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line16_pin<0, (M > 0 ? M - 1 : 0), V - 1>();
+  } else if constexpr (M > 0) {
+    __builtin_amdgcn_sched_group_barrier(0x008, M, 0);
+  }
+#endif
+}
+
+// One k-step of parity E.  X holds the lower-half A operands and B the strips of this k-step on entry, those of
+// the next k-step on exit.  Stage roles as in line_step.
+template <int MTC, int E>
+__device__ __forceinline__ void line16_step(const LineCtx& c, int kb, int ssa, const v4i* __restrict__ cur_a,
+                                            v4i* __restrict__ cur_b, v4i* __restrict__ fill_a, const v4i* __restrict__ nxt_a,
+                                            const v4i* __restrict__ nxt_b, Line16A<MTC>& X, Line16A<MTC>& Y, v4i (&B)[4],
+                                            v4i (&acc)[4][2][4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  // The instructions of a strip stay together (scheduling fences between the strips).  The compiler waits for all
+  // LDS reads at once, so no read may be issued shortly before a wait: strips 0 and 1 of the next k-step are read
+  // in the second half of this one, each after its last use here and two strips before the half ends; strips 2
+  // and 3 are read at the head of the first half of their own k-step, two strips before they are needed.
+  if constexpr (MTC > 0) {
+    B[2] = cur_b[c.b16_off[2]];
+    B[3] = cur_b[c.b16_off[3]];
+    line16_read_a<MTC, E, 1>(c, cur_a, Y);
+    line16_mfma_n<MTC, 0, 0>(X, B, acc);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line_pin<2 + MTC, MTC - 1, 0>();   // the reads two at a time behind the first instructions
+    __builtin_amdgcn_sched_barrier(0);
+    line16_mfma_n<MTC, 0, 1>(X, B, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    line16_mfma_n<MTC, 0, 2>(X, B, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    line16_mfma_n<MTC, 0, 3>(X, B, acc);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt((LINE_LPS & 0xF) | (0x7 << 4) | (0x0 << 8));
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (MTC > 0) {
+    line16_read_a<MTC, 1 - E, 0>(c, nxt_a, X);
+    line16_mfma_n<MTC, 1, 0>(Y, B, acc);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    line16_pin<MTC, MTC - 1, 0>();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  line_load_b(c, kb, cur_b);
+  line_load_a<E>(c, ssa, fill_a);
+  if constexpr (MTC > 0) {
+    B[0] = nxt_b[c.b16_off[0]];
+    line16_mfma_n<MTC, 1, 1>(Y, B, acc);
+    line16_pin<0, MTC, LINE_LPS>();
+    __builtin_amdgcn_sched_barrier(0);
+    B[1] = nxt_b[c.b16_off[1]];
+    line16_mfma_n<MTC, 1, 2>(Y, B, acc);
+    __builtin_amdgcn_sched_barrier(0);
+    line16_mfma_n<MTC, 1, 3>(Y, B, acc);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#endif
+}
+
+template <int MTC>
+__device__ __forceinline__ void line16_k_loop(const LineCtx& c, int nk64, v4i* __restrict__ sa0, v4i* __restrict__ sa1,
+                                              v4i* __restrict__ sa2, v4i* __restrict__ sb0, v4i* __restrict__ sb1,
+                                              v4i* __restrict__ sb2, v4i (&acc)[4][2][4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int last = nk64 - 1, last_ss = nk64 / 2 - 1;
+  Line16A<MTC> X, Y;
+  v4i B[4];
+  __builtin_amdgcn_s_waitcnt((6 & 0xF) | (0x7 << 4) | (0xF << 8));
+  __builtin_amdgcn_s_barrier();
+  line_load_b(c, min(2, last), sb2);
+  if constexpr (MTC > 0) {
+    line16_read_a<MTC, 0, 0>(c, sa0, X);
+    B[0] = sb0[c.b16_off[0]];
+    B[1] = sb0[c.b16_off[1]];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  int k = 0;
+  for (; k + 6 <= nk64; k += 6) {
+    const int ss = k >> 1;
+    line16_step<MTC, 0>(c, min(k + 3, last), min(ss + 2, last_ss), sa0, sb0, sa2, sa0, sb1, X, Y, B, acc);
+    line16_step<MTC, 1>(c, min(k + 4, last), min(ss + 2, last_ss), sa0, sb1, sa2, sa1, sb2, X, Y, B, acc);
+    line16_step<MTC, 0>(c, min(k + 5, last), min(ss + 3, last_ss), sa1, sb2, sa0, sa1, sb0, X, Y, B, acc);
+    line16_step<MTC, 1>(c, min(k + 6, last), min(ss + 3, last_ss), sa1, sb0, sa0, sa2, sb1, X, Y, B, acc);
+    line16_step<MTC, 0>(c, min(k + 7, last), min(ss + 4, last_ss), sa2, sb1, sa1, sa2, sb2, X, Y, B, acc);
+    line16_step<MTC, 1>(c, min(k + 8, last), min(ss + 4, last_ss), sa2, sb2, sa1, sa0, sb0, X, Y, B, acc);
+  }
+  if (k < nk64) {
+    line16_step<MTC, 0>(c, last, last_ss, sa0, sb0, sa2, sa0, sb1, X, Y, B, acc);
+    line16_step<MTC, 1>(c, last, last_ss, sa0, sb1, sa2, sa1, sb2, X, Y, B, acc);
+    if (k + 2 < nk64) {
+      line16_step<MTC, 0>(c, last, last_ss, sa1, sb2, sa0, sa1, sb0, X, Y, B, acc);
+      line16_step<MTC, 1>(c, last, last_ss, sa1, sb0, sa0, sa2, sb1, X, Y, B, acc);
+    }
+  }
+#endif
+}
+
+// From the accumulator layout of the 16x16x64 loop to that of the 32x32x32 loop, in place: registers 8 h + i and
+// 8 h + 4 + i of a 32 x 32 tile (the two strips of a pair, same rows) exchange 16-lane rows.  After the two swaps
+// lane l holds channel l % 32 and rows 8 (r / 4) + 4 (l / 32) + r % 4 in register r, which is what the epilogues
+// and the split-tile hand-over are written for.
+__device__ __forceinline__ void acc16_to_acc32(const v4i (&a16)[4][2][4], v16i (&acc)[4][2]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const auto p = __builtin_amdgcn_permlane16_swap((unsigned)a16[mt][t][2 * h][i], (unsigned)a16[mt][t][2 * h + 1][i], false, false);
+          const auto q = __builtin_amdgcn_permlane32_swap(p[0], p[1], false, false);
+          acc[mt][t][8 * h + i] = (int)q[0];
+          acc[mt][t][8 * h + 4 + i] = (int)q[1];
+        }
 #endif
 }
 
@@ -534,7 +699,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
 // unfused bf16 path); a template parameter so that the fp32 path carries none of that arithmetic.
 // LINES (WN = 4, reduction length a multiple of 128): the line layout of the activation operand and the
 // pinned k loop above; otherwise fragments of 16 rows x 64 bytes and the loop the compiler schedules.
-template <int KIND, int WN, bool BF, bool LINES>
+template <int KIND, int WN, bool BF, bool LINES, bool M16 = false>
 __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   constexpr int BM = 256;
@@ -686,6 +851,15 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
       for (int h = 0; h < 2; ++h) lc.a_off[e][h] = (wm * 128 + r32) * 8 + ((4 * e + 2 * h) ^ gx);
 #pragma unroll
     for (int t = 0; t < 2; ++t) lc.b_off[t] = tile_strip0[t] * WAVE + in_pair;
+    if constexpr (M16) {
+      const int r16 = lane & 15, swz = (r16 >> 1) & 7;
+#pragma unroll
+      for (int e = 0; e < 2; ++e)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) lc.a16_off[e][h] = (wm * 128 + h * 16 + r16) * 8 + ((4 * e + (lane >> 4)) ^ swz);
+#pragma unroll
+      for (int n = 0; n < 4; ++n) lc.b16_off[n] = (tile_strip0[n >> 1] + (n & 1)) * WAVE + lane;
+    }
   } else {
 #pragma unroll
     for (int i = 0; i < AP; ++i) {
@@ -710,22 +884,42 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   }
 
   v16i acc[4][2];
+  if constexpr (!(LINES && M16)) {
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
+        for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0;
+  }
 
   if constexpr (LINES) {
     // one instantiation of the pinned loop per number of row tiles; a wavefront without rows only takes
     // part in the loads and the barriers
-    switch (c.mt_count) {
-      case 4: line_k_loop<4>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-      case 3: line_k_loop<3>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-      case 2: line_k_loop<2>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-      case 1: line_k_loop<1>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
-      default: line_k_loop<0>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+    if constexpr (M16) {
+      v4i a16[4][2][4];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int ch = 0; ch < 4; ++ch) a16[mt][t][ch] = (v4i){0, 0, 0, 0};
+      switch (c.mt_count) {
+        case 4: line16_k_loop<4>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, a16); break;
+        case 3: line16_k_loop<3>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, a16); break;
+        case 2: line16_k_loop<2>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, a16); break;
+        case 1: line16_k_loop<1>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, a16); break;
+        default: line16_k_loop<0>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, a16); break;
+      }
+      acc16_to_acc32(a16, acc);
+    } else {
+      switch (c.mt_count) {
+        case 4: line_k_loop<4>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+        case 3: line_k_loop<3>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+        case 2: line_k_loop<2>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+        case 1: line_k_loop<1>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+        default: line_k_loop<0>(lc, nk64, sa0, sa1, sa2, sb0, sb1, sb2, acc); break;
+      }
     }
   } else {
     // wavefronts whose 128 rows all exist take the loop without tests
@@ -843,6 +1037,7 @@ struct Plan {
 //                          compiled in is refused here, with a message, and the default is used
 //   OMNI_MOE_TILE_WN       2: tile kernel of 256 x 128 instead of 256 x 256
 //   OMNI_MOE_TILE_LINES    0: the 256 x 256 tile kernel keeps the fragment layout of the activation operand
+//   OMNI_MOE_TILE_MFMA16   0: the line-layout tile kernel multiplies with v_mfma_i32_32x32x32_i8 instead of 16x16x64
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
@@ -850,6 +1045,7 @@ struct Plan {
 //                          advance (default 1), bit 1: that of GEMM2 too (measured slower in every geometry)
 struct Tuning {
   int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
+  int tile_mfma16 = 1;
   bool have[3] = {false, false, false};
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
@@ -863,6 +1059,7 @@ Tuning read_tuning() {
   r.force_kernel = geti("OMNI_MOE_FORCE_KERNEL", 0);
   r.tile_wn = geti("OMNI_MOE_TILE_WN", 4);
   r.tile_tail = geti("OMNI_MOE_TILE_TAIL", 1);
+  r.tile_mfma16 = geti("OMNI_MOE_TILE_MFMA16", 1);
   r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
   r.rowq = geti("OMNI_MOE_ROWQ", 0);
   r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
@@ -1040,7 +1237,10 @@ void launch_tile(const GemmArgs& a0, int64_t M_cap, int units, void* tail_ws, si
   dim3 grid((unsigned)nblocks), block(128 * wn);
   const bool bfi = KIND == 1 && (a.flags & OMNI_GEMM1_BF16_INTERMEDIATE);
   if (wn == 4 && tile_lines(a.Kdim)) {
-    if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1, true>), grid, block, 0, st, a);
+    const bool m16 = tuning().tile_mfma16 != 0;
+    if (bfi && m16) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1, true, true>), grid, block, 0, st, a);
+    else if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1, true>), grid, block, 0, st, a);
+    else if (m16) hipLaunchKernelGGL((gemm_pipe<KIND, 4, false, true, true>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((gemm_pipe<KIND, 4, false, true>), grid, block, 0, st, a);
   } else if (wn == 4) {
     if (bfi) hipLaunchKernelGGL((gemm_pipe<KIND, 4, KIND == 1, false>), grid, block, 0, st, a);
