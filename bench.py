@@ -40,8 +40,8 @@ INT8_PEAK = 5.0e15      # op/s, MI355X published dense int8 (256 CU x 8192 op/cl
 # be read from inside a timed run, so these are values of record, labelled with the summary they come from.
 RECORDED_TRAFFIC = {
     ("decode", "gemm1"): (987_888_000, "profiles/decode_gemm1_hbm_traffic.txt"),
-    ("prefill", "gemm1"): (5_613_418_000, "profiles/prefill_gemm1_hbm_traffic.txt"),
-    ("prefill", "gemm2"): (5_043_485_000, "profiles/prefill_gemm1_hbm_traffic.txt"),
+    ("prefill", "gemm1"): (5437806000, "profiles/prefill_gemm1_hbm_traffic.txt"),
+    ("prefill", "gemm2"): (5072506000, "profiles/prefill_gemm1_hbm_traffic.txt"),
 }
 
 SHAPES = {
@@ -475,6 +475,13 @@ def bench_calib(args):
         ops_total = cus * 8 * 8 * iters * 65536.0
         res[f"mfma_i8_{name}_pops"] = ops_total / (ms * 1e-3) / 1e15
         res[f"mfma_i8_{name}_ms"] = ms
+        # the same operands on the tile kernel's pattern (a 128 x 64 piece per wavefront), in both forms of the instruction
+        for form in (32, 16):
+            def run_tile():
+                L.check(lib.omni_diag_mfma_i8_tile_rate(ops_buf.data_ptr(), ops_buf.numel(), form, iters, cus, sink.data_ptr(), st),
+                        "omni_diag_mfma_i8_tile_rate")
+            ms = ev_ms(run_tile, 5)
+            res[f"mfma_i8_tile_pattern_{form}_{name}_pops"] = cus * 8 * iters * 2.0 * 128 * 64 * 64 / (ms * 1e-3) / 1e15
     for tag, (M, K, N) in (("gemm1_shape", (65536, 7168, 4096)), ("gemm2_shape", (65536, 2048, 7168))):
         a = torch.randint(-128, 128, (M, K), generator=g, device=dev, dtype=torch.int8)
         b = torch.randint(-128, 128, (N, K), generator=g, device=dev, dtype=torch.int8).t()   # column-major B

@@ -266,6 +266,15 @@ void omni_moe_reload_tuning(void);
 int omni_diag_mfma_i8_rate(const int8_t* operands, size_t operand_bytes, int iters, int blocks, int32_t* sink,
                            void* stream);
 /*
+ * Diagnostic (no counterpart in the reference): the int8 matrix instruction on the operand pattern of the tile
+ * kernel (a 128 x 64 piece per wavefront, 128 accumulator registers, another operand pair from one instruction
+ * to the next), as v_mfma_i32_32x32x32_i8 (form 32) or v_mfma_i32_16x16x64_i8 (form 16).  One pass of the loop is
+ * 2 x 128 x 64 x 64 op per wavefront either way; `blocks` blocks of 8 wavefronts make `iters` passes.  The caller
+ * times the launch: the two forms sustain different rates on the same operands.
+ */
+int omni_diag_mfma_i8_tile_rate(const int8_t* operands, size_t operand_bytes, int form, int iters, int blocks,
+                                int32_t* sink, void* stream);
+/*
  * Diagnostic (no counterpart in the reference): `blocks` blocks of 256 threads read `bytes` of `buf` once, 16
  * bytes per lane and request, eight requests of a lane in flight, and do nothing else.  The caller times the
  * launch: bytes / time is what the memory system delivers to a kernel that only streams, the practical ceiling

@@ -38,6 +38,7 @@ SIGNATURES = {
     "omni_moe_reload_tuning": (None, []),
     "omni_diag_mfma_i8_rate": (I, [P, c_size_t, I, I, P, P]),
     "omni_diag_hbm_read_rate": (I, [P, c_size_t, I, P, P]),
+    "omni_diag_mfma_i8_tile_rate": (I, [P, c_size_t, I, I, I, P, P]),
     "omni_moe_combine": (I, [P, I, P, P, I, I, I, I, I, P, P, P, P, P]),
     "omni_moe_w8a8_layer": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
     "omni_moe_w8a8_layer_workspace_bytes": (c_size_t, [I, I, I, I, I, I, I]),

@@ -35,6 +35,78 @@ __global__ __launch_bounds__(512, 2) void mfma_i8_rate_kernel(const int8_t* __re
 #endif
 }
 
+// The matrix instruction on the operand pattern of the tile kernel: a 128 x 64 piece per wavefront, 128 accumulator
+// registers, and from one instruction to the next another pair of operands (four row operands x two channel
+// operands per half k-step for 32x32x32, eight x four per k-step for 16x16x64).  Same products, same registers;
+// what differs is how many accumulators an instruction touches per product.
+__global__ __launch_bounds__(512, 2) void mfma_tile32_kernel(const int8_t* __restrict__ operands, int iters, int32_t* __restrict__ sink) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wv = threadIdx.x / WAVE;
+  const v4i* p = (const v4i*)operands + ((blockIdx.x * 8 + wv) % 4) * 16 * WAVE + lane;
+  v4i a[2][4], b[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[h][i] = p[(h * 6 + i) * WAVE];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) b[h][i] = p[(h * 6 + 4 + i) * WAVE];
+  }
+  v16i acc[4][2];
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[m][t][i] = 0;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) acc[m][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[h][m], b[h][t], acc[m][t], 0, 0, 0);
+  }
+  int32_t s = 0;
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s += acc[m][t][i];
+  if (s == 0x7fffffff) sink[0] = s;
+#endif
+}
+__global__ __launch_bounds__(512, 2) void mfma_tile16_kernel(const int8_t* __restrict__ operands, int iters, int32_t* __restrict__ sink) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wv = threadIdx.x / WAVE;
+  const v4i* p = (const v4i*)operands + ((blockIdx.x * 8 + wv) % 4) * 16 * WAVE + lane;
+  v4i a[8], b[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = p[i * WAVE];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b[i] = p[(8 + i) * WAVE];
+  v4i acc[8][4];
+#pragma unroll
+  for (int m = 0; m < 8; ++m)
+#pragma unroll
+    for (int n = 0; n < 4; ++n) acc[m][n] = (v4i){0, 0, 0, 0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int m = 0; m < 8; ++m) acc[m][n] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[m], b[n], acc[m][n], 0, 0, 0);
+  }
+  int32_t s = 0;
+#pragma unroll
+  for (int m = 0; m < 8; ++m)
+#pragma unroll
+    for (int n = 0; n < 4; ++n) s += acc[m][n][0] + acc[m][n][1] + acc[m][n][2] + acc[m][n][3];
+  if (s == 0x7fffffff) sink[0] = s;
+#endif
+}
+
 // Streaming read of a buffer, nothing else: every lane asks for 16 bytes at a time, `DEPTH` requests of a lane in
 // flight, blocks walk the buffer with a grid stride; what arrives is folded into one word so that the loads stay.
 // This is what the memory system delivers to a kernel that only reads: the ceiling of the weight-streaming GEMMs.
@@ -65,6 +137,18 @@ extern "C" int omni_diag_hbm_read_rate(const void* buf, size_t bytes, int blocks
   hipLaunchKernelGGL(hbm_read_rate_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const v4i*)buf,
                      bytes / 16, sink);
   OMNI_CHECK_LAUNCH("diag_hbm_read_rate");
+  return OMNI_OK;
+}
+
+extern "C" int omni_diag_mfma_i8_tile_rate(const int8_t* operands, size_t operand_bytes, int form, int iters, int blocks,
+                                           int32_t* sink, void* stream) {
+  if (!operands || !sink || iters <= 0 || blocks <= 0) OMNI_FAIL(OMNI_E_INVALID, "diag_mfma_i8_tile_rate: bad arguments");
+  if (form != 16 && form != 32) OMNI_FAIL(OMNI_E_INVALID, "diag_mfma_i8_tile_rate: form %d (16: 16x16x64, 32: 32x32x32)", form);
+  if (operand_bytes < (size_t)4 * 16 * WAVE * 16) OMNI_FAIL(OMNI_E_INVALID, "diag_mfma_i8_tile_rate: operand buffer below 64 KiB");
+  if ((uintptr_t)operands % 16) OMNI_FAIL(OMNI_E_INVALID, "diag_mfma_i8_tile_rate: operands must be 16-byte aligned");
+  if (form == 32) hipLaunchKernelGGL(mfma_tile32_kernel, dim3((unsigned)blocks), dim3(512), 0, (hipStream_t)stream, operands, iters, sink);
+  else hipLaunchKernelGGL(mfma_tile16_kernel, dim3((unsigned)blocks), dim3(512), 0, (hipStream_t)stream, operands, iters, sink);
+  OMNI_CHECK_LAUNCH("diag_mfma_i8_tile_rate");
   return OMNI_OK;
 }
 
