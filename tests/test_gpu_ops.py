@@ -270,8 +270,8 @@ def _tile_outputs(ops, lay_dev, xq, xs, p, K, H, I, M_cap):
 ])
 def test_tile_layouts_give_the_same_bits(ops, tuning, T, K, n_local, E, H, I):
     """The tile kernel has two layouts of the activation operand in LDS (whole 128-byte lines with the pinned
-    k loop, the default where it applies, and 16-row fragments) and two tile widths: all of them give the bits
-    of the oracle."""
+    k loop, the default where it applies, and 16-row fragments), two forms of the matrix instruction in the line
+    layout (16x16x64, the default, and 32x32x32) and two tile widths: all of them give the bits of the oracle."""
     from omni_infer_amd import _lib as L
     lay, xq, xs, ids, w = _grouped_case(T, K, n_local, E, H, I, 300 + T)
     d = lay.to_device()
@@ -281,19 +281,21 @@ def test_tile_layouts_give_the_same_bits(ops, tuning, T, K, n_local, E, H, I):
     p = ops.moe_permute(ids.cuda(), 0, n_local, L.OMNI_IDX_TOKEN_MAJOR)
     M_cap = T * K
     seen = {}
-    for tag, env in (("lines", dict(OMNI_MOE_TILE_LINES=1, OMNI_MOE_TILE_WN=4)),
+    for tag, env in (("lines", dict(OMNI_MOE_TILE_LINES=1, OMNI_MOE_TILE_WN=4, OMNI_MOE_TILE_MFMA16=1)),
+                     ("lines32", dict(OMNI_MOE_TILE_LINES=1, OMNI_MOE_TILE_WN=4, OMNI_MOE_TILE_MFMA16=0)),
                      ("frags", dict(OMNI_MOE_TILE_LINES=0, OMNI_MOE_TILE_WN=4)),
                      ("narrow", dict(OMNI_MOE_TILE_LINES=1, OMNI_MOE_TILE_WN=2))):
         tuning(OMNI_MOE_FORCE_KERNEL=2, **env)
         name = ops.gemm_kernel_name(1, T, K, n_local, 0, M_cap, H, I)
-        assert name == {"lines": "gemm_pipe<1,4,lines>", "frags": "gemm_pipe<1,4,frags>", "narrow": "gemm_pipe<1,2,frags>"}[tag]
+        assert name == {"lines": "gemm_pipe<1,4,lines>", "lines32": "gemm_pipe<1,4,lines>", "frags": "gemm_pipe<1,4,frags>",
+                        "narrow": "gemm_pipe<1,2,frags>"}[tag]
         seen[tag] = _tile_outputs(ops, d, xq.cuda(), xs.cuda(), p, K, H, I, M_cap)
     h_q, h_s, acc1 = seen["lines"][:3]
     _eq(acc1[:m], st["acc1"], "GEMM1 int32 accumulators")
     _eq(h_s[:m], st["h_s"], "stage-2 scales")
     _eq(h_q[:m], st["h_q"], "stage-2 int8 activations")
     _eq(seen["lines"][4][:m], st["acc2"], "GEMM2 int32 accumulators")
-    for tag in ("frags", "narrow"):
+    for tag in ("lines32", "frags", "narrow"):
         for a, b, what in zip(seen[tag], seen["lines"], ("h_q", "h_s", "acc1", "rows f32", "acc2", "rows bf16", "acc2")):
             assert torch.equal(a[:m], b[:m]), f"{what}: {tag} differs from the line layout"
 
