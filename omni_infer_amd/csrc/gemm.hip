@@ -22,7 +22,8 @@
 //                is small and shared by the four wavefronts of a block through LDS.
 //   gemm_pipe    many rows per group (prefill): 256 x 256 (or 256 x 128) block tiles, A and B both
 //                loaded straight into LDS (global_load_lds) through a three-stage ring, each
-//                wavefront a 128 x 64 sub-tile on the 32x32x32 MFMA.
+//                wavefront a 128 x 64 sub-tile: on the 16x16x64 MFMA in the line layout (the default
+//                wherever it applies), on the 32x32x32 MFMA in the fragment layout.
 //
 // GEMM1 pairs gate channel n with up channel I + n in the same lane so SwiGLU needs no exchange.
 // Its epilogue writes y = silu(gate) * up in fp32 to a scratch matrix; a row kernel
@@ -128,7 +129,8 @@ __global__ __launch_bounds__(NTH) void swiglu_quant_rows(GemmArgs a, int8_t* __r
 // gemm_pipe: large row counts.  Block tile 256 rows x 128 channels (GEMM1: 64 gate + 64 up),
 // four wavefronts as 2 (rows) x 2 (channels), each a 128 x 64 sub-tile held as 4 x 2 accumulator
 // tiles of v_mfma_i32_32x32x32_i8 (a single wavefront issues the 32x32x32 form at nearly the
-// full MFMA rate, the 16x16x64 form at about half of it).
+// full MFMA rate, the 16x16x64 form at about half of it; with the two wavefronts per SIMD of this
+// kernel both forms issue at the full rate, and the line-layout loop further down uses 16x16x64).
 //   Operands go from global memory straight into LDS (global_load_lds, 16 bytes per lane, no
 //   register staging) through a three-stage ring: while stage s is multiplied, stages s+1 and s+2
 //   are in flight.  A wavefront's load instruction moves one 1 KiB fragment of 16 rows (or 16
