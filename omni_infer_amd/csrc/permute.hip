@@ -40,19 +40,35 @@ __device__ __forceinline__ int bucket_of(int id, int lo, int G) {
   return (e >= 0 && e < G) ? e : G;
 }
 
+// The buckets of a thread's assignments of the chunk, all requested at once (the passes below depend on each
+// other through the histogram, so loads inside them would be paid one latency at a time): bk[j] is the bucket of
+// assignment (w * passes + j) * 64 + lane, -1 past the end.  MP bounds the passes of a chunk.
+template <int MP>
+__device__ __forceinline__ void load_buckets(const PermArgs& a, int base, int len, int passes, int (&bk)[MP]) {
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int j = 0; j < MP; ++j) {
+    const int i = (w * passes + j) * WAVE + lane;
+    bk[j] = (j < passes && i < len) ? bucket_of(a.ids[base + i], a.lo, a.G) : -1;
+  }
+}
+
 // Ranks the chunk [base, base+len): lrank[i] = number of earlier assignments of the same bucket
 // inside the same wavefront's part; whist[w][b] = count of bucket b in wavefront w's part.
-__device__ __forceinline__ void rank_chunk(const PermArgs& a, int base, int len, int passes, int (*whist)[NB],
-                                           int* lrank) {
+template <int MP>
+__device__ __forceinline__ void rank_chunk(const PermArgs& a, int len, int passes, int (*whist)[NB], int* lrank,
+                                           const int (&bk)[MP]) {
   const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
   for (int i = threadIdx.x; i < 4 * NB; i += 256) (&whist[0][0])[i] = 0;
   __syncthreads();
   const int nbits = 32 - __clz(a.G);
   const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  for (int j = 0; j < passes; ++j) {
+#pragma unroll
+  for (int j = 0; j < MP; ++j) {
+    if (j >= passes) break;
     int i = (w * passes + j) * WAVE + lane;
-    bool valid = i < len;
-    int b = valid ? bucket_of(a.ids[base + i], a.lo, a.G) : 0;
+    bool valid = bk[j] >= 0;
+    int b = valid ? bk[j] : 0;
     uint64_t peers = __ballot(valid);
     for (int bit = 0; bit < nbits; ++bit) {
       uint64_t m = __ballot((b >> bit) & 1);
@@ -78,13 +94,16 @@ __device__ __forceinline__ int src_index(const PermArgs& a, int p) {
 }
 
 // Scatter of the chunk, given for every bucket the slot of the chunk's first assignment of it.
-__device__ __forceinline__ void scatter_chunk(const PermArgs& a, int base, int len, int passes, int (*whist)[NB],
-                                              const int* lrank, const int* bucket_slot0) {
+template <int MP>
+__device__ __forceinline__ void scatter_chunk(const PermArgs& a, int base, int passes, int (*whist)[NB],
+                                              const int* lrank, const int* bucket_slot0, const int (&bk)[MP]) {
   const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
-  for (int j = 0; j < passes; ++j) {
+#pragma unroll
+  for (int j = 0; j < MP; ++j) {
+    if (j >= passes) break;
     int i = (w * passes + j) * WAVE + lane;
-    if (i < len) {
-      int b = bucket_of(a.ids[base + i], a.lo, a.G);
+    if (bk[j] >= 0) {
+      int b = bk[j];
       int slot = bucket_slot0[b] + lrank[i];
       for (int ww = 0; ww < w; ++ww) slot += whist[ww][b];
       int src = src_index(a, base + i);
@@ -123,8 +142,10 @@ __device__ __forceinline__ void permute_single_body(const PermArgs& a) {
   __shared__ int tot[NB];
   __shared__ int off[NB + 1];
   const int passes = (a.n + 255) / 256;
+  int bk[CH_SINGLE / 256];
+  load_buckets(a, 0, a.n, passes, bk);
   clear_words(a);
-  rank_chunk(a, 0, a.n, passes, whist, lrank);
+  rank_chunk(a, a.n, passes, whist, lrank, bk);
   const int nb = a.G + 1;
   for (int b = threadIdx.x; b < nb; b += 256) tot[b] = whist[0][b] + whist[1][b] + whist[2][b] + whist[3][b];
   __syncthreads();
@@ -135,7 +156,7 @@ __device__ __forceinline__ void permute_single_body(const PermArgs& a) {
     a.offsets[b] = off[b];
   }
   if (threadIdx.x == 0) a.offsets[a.G] = off[a.G];
-  scatter_chunk(a, 0, a.n, passes, whist, lrank, off);
+  scatter_chunk(a, 0, passes, whist, lrank, off, bk);
 }
 
 __global__ __launch_bounds__(256) void permute_single(PermArgs a) { permute_single_body(a); }
@@ -156,7 +177,9 @@ __global__ __launch_bounds__(256) void permute_count(PermArgs a) {
   __shared__ int lrank[CH_MULTI];
   const int base = blockIdx.x * CH_MULTI;
   const int len = min(CH_MULTI, a.n - base);
-  rank_chunk(a, base, len, CH_MULTI / 256, whist, lrank);
+  int bk[CH_MULTI / 256];
+  load_buckets(a, base, len, CH_MULTI / 256, bk);
+  rank_chunk(a, len, CH_MULTI / 256, whist, lrank, bk);
   for (int b = threadIdx.x; b <= a.G; b += 256)
     a.blk_hist[(size_t)blockIdx.x * NB + b] = whist[0][b] + whist[1][b] + whist[2][b] + whist[3][b];
 }
@@ -200,11 +223,13 @@ __global__ __launch_bounds__(256) void permute_scatter(PermArgs a) {
   __shared__ int slot0[NB];
   const int base = blockIdx.x * CH_MULTI;
   const int len = min(CH_MULTI, a.n - base);
-  rank_chunk(a, base, len, CH_MULTI / 256, whist, lrank);
+  int bk[CH_MULTI / 256];
+  load_buckets(a, base, len, CH_MULTI / 256, bk);
+  rank_chunk(a, len, CH_MULTI / 256, whist, lrank, bk);
   for (int b = threadIdx.x; b <= a.G; b += 256)
     slot0[b] = a.blk_hist[(size_t)a.nblk * NB + b] + a.blk_hist[(size_t)blockIdx.x * NB + b];
   __syncthreads();
-  scatter_chunk(a, base, len, CH_MULTI / 256, whist, lrank, slot0);
+  scatter_chunk(a, base, CH_MULTI / 256, whist, lrank, slot0, bk);
 }
 
 struct GatherArgs {
