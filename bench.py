@@ -107,6 +107,15 @@ def make_inputs(cfg, dev):
     return x.to(torch.bfloat16).to(dev), logits.to(dev), bias.to(dev)
 
 
+def noaux_tc_routing(cfg):
+    """The routing arguments of npu_moe_gating_top_k as the reference calls it (layer.py:341-351): sigmoid scores,
+    bias for the selection only, groups ranked by the sum of their two best, weights renormalised and scaled."""
+    from omni_infer_amd import _lib as L
+    return dict(top_k=cfg["K"], n_group=cfg["n_group"], topk_group=cfg["topk_group"], score_fn="sigmoid",
+                group_mode=L.OMNI_GROUP_TOP2SUM, masked_fill_zero=False, weight_from_c=False, renorm=True,
+                scale=cfg["scale"], eps=1e-20)
+
+
 def algorithmic_bytes_layer(cfg, groups_active):
     H, I, T = cfg["H"], cfg["I"], cfg["T"]
     w = groups_active * (H * 2 * I + I * H)
@@ -248,13 +257,17 @@ def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_ste
     workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
 
+    topk_w = torch.empty(T, K, dtype=torch.float32, device=dev)
+    topk_ids = torch.empty(T, K, dtype=torch.int32, device=dev)
+
     def step(i):
+        # router (npu_moe_gating_top_k as called at layer.py:341-351) and layer in one library call
         ws = sets[i % len(sets)]
-        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
-                                             cfg["scale"], 1e-20)
-        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
-                                  (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out,
-                                  rows_dtype=rows_dtype)
+        return ops.moe_w8a8_layer_routed(x, None, logits, bias, lo=0, hi=n_local, w13_packed=ws.w13, w13_scale=ws.s13,
+                                         w2_packed=ws.w2, w2_scale=ws.s2,
+                                         shared=(ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace,
+                                         out=out, rows_dtype=rows_dtype, topk_w=topk_w, topk_ids=topk_ids,
+                                         **noaux_tc_routing(cfg))[0]
 
     ms, wall_ms = time_steps(step, steps, warmup)
     spread = single_step_spread(step, min(50, steps))
@@ -357,13 +370,17 @@ def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
     workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
 
+    topk_w = torch.empty(T, K, dtype=torch.float32, device=dev)
+    topk_ids = torch.empty(T, K, dtype=torch.int32, device=dev)
+
     def step(i):
+        # router (npu_moe_gating_top_k as called at layer.py:341-351) and layer in one library call
         ws = sets[i % len(sets)]
-        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
-                                             cfg["scale"], 1e-20)
-        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2,
-                                  (ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace, out=out,
-                                  rows_dtype=rows_dtype)
+        return ops.moe_w8a8_layer_routed(x, None, logits, bias, lo=0, hi=n_local, w13_packed=ws.w13, w13_scale=ws.s13,
+                                         w2_packed=ws.w2, w2_scale=ws.s2,
+                                         shared=(ws.sh13, ws.sh_s13, ws.sh2, ws.sh_s2), H=H, I=I, workspace=workspace,
+                                         out=out, rows_dtype=rows_dtype, topk_w=topk_w, topk_ids=topk_ids,
+                                         **noaux_tc_routing(cfg))[0]
 
     ms, _ = time_steps(step, steps, warmup)
 
@@ -371,10 +388,10 @@ def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
         # the reference runs the shared expert on the rank's own tokens before the all-gather (deepseek_moe.py:244):
         # on the gathered tokens only the routed experts are computed
         ws = sets[i % len(sets)]
-        w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1,
-                                             cfg["scale"], 1e-20)
-        return ops.moe_w8a8_layer(x, None, w, ids, 0, n_local, ws.w13, ws.s13, ws.w2, ws.s2, None, H=H, I=I,
-                                  workspace=workspace, out=out, rows_dtype=rows_dtype)
+        return ops.moe_w8a8_layer_routed(x, None, logits, bias, lo=0, hi=n_local, w13_packed=ws.w13, w13_scale=ws.s13,
+                                         w2_packed=ws.w2, w2_scale=ws.s2, shared=None, H=H, I=I, workspace=workspace,
+                                         out=out, rows_dtype=rows_dtype, topk_w=topk_w, topk_ids=topk_ids,
+                                         **noaux_tc_routing(cfg))[0]
 
     ms_routed, _ = time_steps(step_routed_only, steps, warmup)
     w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)

@@ -317,6 +317,24 @@ int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, con
 size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared, int rows_dtype);
 
 /*
+ * Router and layer in one call: FusedMoE.select_experts followed by the quant method's apply, the two steps
+ * of a MoE block between the gate projection and the sum with the shared expert (deepseek_moe.py:253-263,
+ * 329-339; layer.py:301-365).  The results are those of omni_moe_route followed by omni_moe_w8a8_layer, bit
+ * for bit: the routing arguments (logits .. eps) mean what they mean for omni_moe_route, topk_w [T,K] fp32 and
+ * topk_ids [T,K] int32 are outputs here and hold the routing when the call's work is done, everything else is
+ * as for omni_moe_w8a8_layer, workspace size included.  Small calls (bf16 tokens, T*K <= 4096, H <= 8192) route,
+ * quantise and sort in a single launch; other calls run the router's own launch first.
+ */
+int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const float* x_scale_in, const float* logits,
+                               const float* bias, int E, int n_group, int topk_group, int score_fn, int group_mode,
+                               int masked_fill_zero, int weight_from_c, int renorm, float scale, float eps,
+                               float* topk_w, int32_t* topk_ids, int T, int K, int lo, int hi,
+                               const int8_t* w13_packed, const float* w13_scale, const int8_t* w2_packed,
+                               const float* w2_scale, const int8_t* sh13_packed, const float* sh13_scale,
+                               const int8_t* sh2_packed, const float* sh2_scale, int H, int I, int rows_dtype,
+                               void* out_bf16, void* workspace, size_t ws_bytes, void* stream);
+
+/*
  * The same layer on the library's own scratch.  No counterpart in the reference: it is for callers
  * that cannot allocate device memory or hold a workspace (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  Arguments and results are those of omni_moe_w8a8_layer

@@ -18,7 +18,7 @@ void omni_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 extern "C" const char* omni_moe_last_error(void) { return g_err; }
-extern "C" int omni_moe_abi_version(void) { return 5; }
+extern "C" int omni_moe_abi_version(void) { return 6; }
 
 namespace {
 
@@ -230,12 +230,15 @@ extern "C" size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local,
   return layer_layout(T, K, n_local, H, I, with_shared, rows_dtype).total;
 }
 
-extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
-                                   const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
-                                   const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
-                                   const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
-                                   const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16,
-                                   void* workspace, size_t ws_bytes, void* stream) {
+namespace {
+// The layer.  With `route` the routing is part of the call: topk_w and topk_ids are route's outputs, written before
+// anything reads them (by the first launch when the call is small enough for the kernel that routes, quantises
+// and sorts at once, by a routing launch of its own otherwise).
+int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w, const int32_t* topk_ids,
+               const OmniRouteParams* route, int T, int K, int lo, int hi, const int8_t* w13_packed,
+               const float* w13_scale, const int8_t* w2_packed, const float* w2_scale, const int8_t* sh13_packed,
+               const float* sh13_scale, const int8_t* sh2_packed, const float* sh2_scale, int H, int I, int rows_dtype,
+               void* out_bf16, void* workspace, size_t ws_bytes, void* stream) {
   if (T < 0 || K <= 0 || hi <= lo || H <= 0 || I <= 0) OMNI_FAIL(OMNI_E_INVALID, "layer: bad sizes");
   if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "layer: rows_dtype %d", rows_dtype);
   if (T == 0) return OMNI_OK;
@@ -261,7 +264,25 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
   int cnt_words = 0;
   size_t tail_bytes = 0;
   void* const tail = omni_tile_tail_area(T, K, G, extra, L.M_cap, H, I, ws + L.g1_ws, L.g1_bytes, &cnt_words, &tail_bytes);
-  if (x_dtype != -1) {
+  bool routed = route == nullptr;
+  if (route != nullptr && x_dtype == OMNI_DT_BF16) {
+    // routing, quantisation and sort in one launch when the call is small
+    rc = omni_route_quant_permute_fused(route, x, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), K, lo, hi, sorted_src,
+                                        src_to_dst, (int32_t*)(ws + L.counts), offsets, (int32_t*)tail, cnt_words, stream);
+    if (rc < 0) return rc;
+    routed = sorted = rc == 0;
+    if (sorted) {
+      xq = (const int8_t*)(ws + L.x_q);
+      xs = (const float*)(ws + L.x_s);
+    }
+  }
+  if (!routed) {
+    rc = omni_moe_route(route->logits, route->bias, T, route->E, route->n_group, route->topk_group, K, route->score_fn,
+                        route->group_mode, route->masked_fill_zero, route->weight_from_c, route->renorm, route->scale,
+                        route->eps, route->topk_w, route->topk_ids, stream);
+    if (rc) return rc;
+  }
+  if (x_dtype != -1 && !sorted) {
     // the quantisation and the sort do not depend on each other: one launch when both are small
     rc = 1;
     if (x_dtype == OMNI_DT_BF16)
@@ -296,6 +317,39 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
   return omni_moe_combine(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
                           nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,
                           stream);
+}
+}  // namespace
+
+extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
+                                   const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
+                                   const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
+                                   const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
+                                   const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16,
+                                   void* workspace, size_t ws_bytes, void* stream) {
+  return layer_impl(x, x_dtype, x_scale_in, topk_w, topk_ids, nullptr, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
+                    w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, workspace,
+                    ws_bytes, stream);
+}
+
+extern "C" int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const float* x_scale_in, const float* logits,
+                                          const float* bias, int E, int n_group, int topk_group, int score_fn,
+                                          int group_mode, int masked_fill_zero, int weight_from_c, int renorm,
+                                          float scale, float eps, float* topk_w, int32_t* topk_ids, int T, int K, int lo,
+                                          int hi, const int8_t* w13_packed, const float* w13_scale,
+                                          const int8_t* w2_packed, const float* w2_scale, const int8_t* sh13_packed,
+                                          const float* sh13_scale, const int8_t* sh2_packed, const float* sh2_scale,
+                                          int H, int I, int rows_dtype, void* out_bf16, void* workspace, size_t ws_bytes,
+                                          void* stream) {
+  if (T < 0 || E <= 0 || K <= 0) OMNI_FAIL(OMNI_E_INVALID, "layer_routed: bad sizes T=%d E=%d K=%d", T, E, K);
+  if (T == 0) return OMNI_OK;
+  if (!logits || !topk_w || !topk_ids) OMNI_FAIL(OMNI_E_INVALID, "layer_routed: null pointer");
+  const int rc = omni_route_check("layer_routed", T, E, n_group, topk_group, K, score_fn);
+  if (rc) return rc;
+  const OmniRouteParams rp{logits, bias, E, n_group, topk_group, score_fn, group_mode, masked_fill_zero, weight_from_c,
+                           renorm, scale, eps, topk_w, topk_ids};
+  return layer_impl(x, x_dtype, x_scale_in, topk_w, topk_ids, &rp, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
+                    w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, workspace,
+                    ws_bytes, stream);
 }
 
 // ---------------------------------------------------------------- whole layer on the library's own scratch

@@ -37,6 +37,22 @@ void omni_set_error(const char* fmt, ...);
 int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float* scale, const int32_t* topk_ids, int K,
                              int lo, int hi, int idx_mode, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
                              int32_t* offsets, int32_t* zero_words, int zero_n, void* stream);
+// library-internal: the router's arguments as the whole-layer entry hands them on; topk_w and topk_ids are outputs
+struct OmniRouteParams {
+  const float* logits;
+  const float* bias;
+  int E, n_group, topk_group, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm;
+  float scale, eps;
+  float* topk_w;
+  int32_t* topk_ids;
+};
+// library-internal: the argument checks of omni_moe_route (route.hip)
+int omni_route_check(const char* what, int T, int E, int n_group, int topk_group, int K, int score_fn);
+// library-internal: routing, bf16 row quantisation and assignment sort in one launch (permute.hip); 1 = not
+// applicable.  zero_words as above.
+int omni_route_quant_permute_fused(const OmniRouteParams* rp, const void* x_bf16, int T, int H, int8_t* q, float* scale,
+                                   int K, int lo, int hi, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
+                                   int32_t* offsets, int32_t* zero_words, int zero_n, void* stream);
 // library-internal: omni_moe_permute that also clears zero_words (in its single-block kernel)
 int omni_moe_permute_clearing(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode, int32_t* sorted_src,
                               int32_t* src_to_dst, int32_t* counts, int32_t* offsets, void* workspace, size_t ws_bytes,

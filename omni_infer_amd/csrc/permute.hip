@@ -8,8 +8,11 @@
 // An exclusive prefix over wavefronts, blocks and buckets then gives every assignment its slot.
 // Small inputs (<= 4096 assignments) are sorted by one block in one launch; larger ones take a
 // count launch, a one-block scan launch and a scatter launch.
+#include <atomic>
+#include <mutex>
 #include "common.h"
 #include "quant_rows.h"
+#include "route_body.h"
 
 namespace {
 
@@ -172,6 +175,45 @@ __global__ __launch_bounds__(256) void quant_permute_small(const void* __restric
   else permute_single_body(a);
 }
 
+// One launch for the three first steps of a small layer call: blocks [0, ceil(T/4)) route four tokens each (one
+// per wavefront), the other T blocks quantise one bf16 token row each, and the routing block that finishes last
+// sorts the assignments.  `arrive` counts the routing blocks that are done.  It is zero when the kernel starts and
+// the sorting block sets it back to zero, so no launch ever has to clear it.  The hand-over is the one of the
+// split tiles of the grouped GEMM: every wavefront waits for its stores, the block meets at a barrier, one
+// thread counts in with a device-scope acquire-release add (the release half makes the block's stores visible to
+// the device, the acquire half of the last add makes everybody else's visible to the sorting block).  No block
+// waits for another.
+template <int MAXV, int V>
+__global__ __launch_bounds__(256) void route_quant_permute_small(const void* __restrict__ x, int64_t rows, int cols,
+                                                                 int8_t* __restrict__ q, float* __restrict__ scale,
+                                                                 RouteArgs r, PermArgs a, int* arrive) {
+  __shared__ float red[4];
+  __shared__ int s_last;
+  const int route_blocks = (r.T + 3) / 4;
+  if ((int)blockIdx.x >= route_blocks) {
+    quant_row_vec_body<OMNI_DT_BF16, MAXV>(x, (int64_t)blockIdx.x - route_blocks, cols, cols, q, scale, red);
+    return;
+  }
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int t = (int)blockIdx.x * 4 + threadIdx.x / WAVE;
+  if (t < r.T) {  // the same for a whole wavefront
+    float s[V], bias[V];
+    bool in[V];
+    route_load_bias<V>(r, lane, bias);
+    route_load_logits<V>(r, t, lane, s, in);
+    route_token<V>(r, t, lane, s, in, bias);
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    s_last = (__hip_atomic_fetch_add(arrive, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == route_blocks - 1);
+    if (s_last) __hip_atomic_store(arrive, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  permute_single_body(a);
+}
+
 __global__ __launch_bounds__(256) void permute_count(PermArgs a) {
   __shared__ int whist[4][NB];
   __shared__ int lrank[CH_MULTI];
@@ -322,6 +364,80 @@ int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float*
   else if (H <= 8 * 256 * 2) hipLaunchKernelGGL(quant_permute_small<2>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
   else hipLaunchKernelGGL(quant_permute_small<4>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
   OMNI_CHECK_LAUNCH("quant_permute");
+  return OMNI_OK;
+}
+
+// ---- arrival counters of the kernel that routes, quantises and sorts
+// A file-scope device array, zero when the module is loaded; every GPU holds its own copy at its own address (the
+// array's name is only a host-side handle: the device address is asked for once per device).  Calls take the
+// counters in turn, so calls that overlap on one GPU (other streams) use different ones as long as fewer than
+// ARRIVE_SLOTS of them are in flight; each kernel leaves its counter at zero.
+namespace {
+constexpr int ARRIVE_SLOTS = 256;
+static __device__ int arrive_counters[ARRIVE_SLOTS];
+constexpr int ARRIVE_MAX_DEVICES = 64;
+int* g_arrive_ptr[ARRIVE_MAX_DEVICES];
+std::mutex g_arrive_mutex;
+std::atomic<unsigned> g_arrive_next{0};
+
+int next_arrive_counter(int** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ARRIVE_MAX_DEVICES)
+    OMNI_FAIL(OMNI_E_LAUNCH, "route_quant_permute: no current device (or device index >= %d)", ARRIVE_MAX_DEVICES);
+  int* base;
+  {
+    std::lock_guard<std::mutex> lock(g_arrive_mutex);
+    if (g_arrive_ptr[dev] == nullptr) {
+      void* ptr = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(arrive_counters));
+      if (e != hipSuccess || ptr == nullptr)
+        OMNI_FAIL(OMNI_E_LAUNCH, "route_quant_permute: hipGetSymbolAddress(arrive_counters): %s", hipGetErrorString(e));
+      g_arrive_ptr[dev] = (int*)ptr;
+    }
+    base = g_arrive_ptr[dev];
+  }
+  *out = base + g_arrive_next.fetch_add(1, std::memory_order_relaxed) % ARRIVE_SLOTS;
+  return OMNI_OK;
+}
+}  // namespace
+
+// Internal to the library (the whole-layer entry uses it): route, quantise bf16 rows and sort the assignments in
+// one launch.  Returns 1 without launching when the shapes do not fit that kernel.  The routing arguments have
+// been checked by the caller (omni_route_check).
+int omni_route_quant_permute_fused(const OmniRouteParams* rp, const void* x_bf16, int T, int H, int8_t* q, float* scale,
+                                   int K, int lo, int hi, int32_t* sorted_src, int32_t* src_to_dst, int32_t* counts,
+                                   int32_t* offsets, int32_t* zero_words, int zero_n, void* stream) {
+  const int G = hi - lo;
+  const int64_t n = (int64_t)T * K;
+  if (T <= 0 || n > CH_SINGLE || G > GMAX || H % 8 != 0 || H > 8 * 256 * 4) return 1;
+  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((size_t)H * 2) % 16 != 0) return 1;
+  int* arrive = nullptr;
+  const int rc = next_arrive_counter(&arrive);
+  if (rc) return rc;
+  RouteArgs r{rp->logits, nullptr, 0, 1, 0, nullptr, 0, rp->bias, T, rp->E, rp->n_group, rp->topk_group, K, rp->score_fn,
+              rp->group_mode, rp->masked_fill_zero, rp->weight_from_c, rp->renorm, rp->scale, rp->eps, rp->topk_w,
+              rp->topk_ids};
+  PermArgs a{rp->topk_ids, (int)n, T, K, lo, G, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, counts, offsets, nullptr, 0,
+             zero_words, zero_words ? zero_n : 0};
+  dim3 grid((unsigned)(T + (T + 3) / 4)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int V = (rp->E + 63) / 64;
+  const int MV = H <= 8 * 256 ? 1 : (H <= 8 * 256 * 2 ? 2 : 4);
+#define RQP_LAUNCH(MAXV, VV) \
+  hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, r, a, arrive)
+#define RQP_V(MAXV)                      \
+  do {                                   \
+    if (V <= 1) RQP_LAUNCH(MAXV, 1);     \
+    else if (V <= 2) RQP_LAUNCH(MAXV, 2); \
+    else if (V <= 4) RQP_LAUNCH(MAXV, 4); \
+    else RQP_LAUNCH(MAXV, 8);            \
+  } while (0)
+  if (MV == 1) RQP_V(1);
+  else if (MV == 2) RQP_V(2);
+  else RQP_V(4);
+#undef RQP_V
+#undef RQP_LAUNCH
+  OMNI_CHECK_LAUNCH("route_quant_permute");
   return OMNI_OK;
 }
 

@@ -413,6 +413,60 @@ def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: tor
     return out
 
 
+def moe_w8a8_layer_routed(x: torch.Tensor, x_scale: Optional[torch.Tensor], logits: torch.Tensor,
+                          bias: Optional[torch.Tensor], top_k: int, n_group: int, topk_group: int, score_fn: str,
+                          group_mode: int, masked_fill_zero: bool, weight_from_c: bool, renorm: bool, scale: float,
+                          eps: float, lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None,
+                          H: int = 0, I: int = 0, workspace: Optional[torch.Tensor] = None,
+                          out: Optional[torch.Tensor] = None, rows_dtype: torch.dtype = torch.float32,
+                          topk_w: Optional[torch.Tensor] = None, topk_ids: Optional[torch.Tensor] = None):
+    """``moe_route`` followed by ``moe_w8a8_layer`` in one library call (``FusedMoE.select_experts`` and the
+    quant method's ``apply``: deepseek_moe.py:253-263; layer.py:301-365), the same bits as the two calls.  Small
+    calls route, quantise and sort in a single launch.  Returns (out, topk_w, topk_ids)."""
+    _need_gpu(x, logits, bias)
+    if logits.dim() != 2:
+        raise ValueError("router logits must be [T, E]")
+    logits = logits.float().contiguous()
+    T, E = logits.shape
+    if x.shape[0] != T:
+        raise ValueError("one row of logits per token")
+    if bias is not None:
+        bias = bias.float().contiguous()
+        if bias.numel() != E:
+            raise ValueError("bias must have one entry per expert")
+    fn = {"softmax": L.OMNI_SCORE_SOFTMAX, "sigmoid": L.OMNI_SCORE_SIGMOID}.get(score_fn)
+    if fn is None:
+        raise ValueError(f"Unsupported scoring function: {score_fn}")
+    if rows_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("rows_dtype must be torch.float32 or torch.bfloat16")
+    dev = x.device
+    x = x.contiguous()
+    K = int(top_k)
+    if topk_w is None:
+        topk_w = torch.empty(T, K, dtype=torch.float32, device=dev)
+    if topk_ids is None:
+        topk_ids = torch.empty(T, K, dtype=torch.int32, device=dev)
+    if (topk_w.dtype != torch.float32 or topk_ids.dtype != torch.int32 or tuple(topk_w.shape) != (T, K) or
+            tuple(topk_ids.shape) != (T, K) or not topk_w.is_contiguous() or not topk_ids.is_contiguous()):
+        raise ValueError("topk_w must be a contiguous fp32 [T, K] tensor and topk_ids a contiguous int32 one")
+    x_dtype = -1 if x.dtype == torch.int8 else _DT[x.dtype]
+    sh = shared if shared is not None else (None, None, None, None)
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, hi - lo, H, I, int(shared is not None), _DT[rows_dtype])
+    if workspace is None or workspace.numel() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    rc = L.lib().omni_moe_w8a8_layer_routed(_ptr(x), x_dtype, _ptr(x_scale), _ptr(logits), _ptr(bias), E, int(n_group),
+                                            int(topk_group), fn, int(group_mode), int(masked_fill_zero),
+                                            int(weight_from_c), int(renorm), float(scale), float(eps), _ptr(topk_w),
+                                            _ptr(topk_ids), T, K, lo, hi, _ptr(w13_packed), _ptr(w13_scale),
+                                            _ptr(w2_packed), _ptr(w2_scale), _ptr(sh[0]), _ptr(sh[1]), _ptr(sh[2]),
+                                            _ptr(sh[3]), H, I, _DT[rows_dtype], _ptr(out), _ptr(workspace),
+                                            workspace.numel(), _stream())
+    L.check(rc, "omni_moe_w8a8_layer_routed")
+    return out, topk_w, topk_ids
+
+
 def moe_w8a8_layer_static(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: torch.Tensor, topk_ids: torch.Tensor,
                           lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None, H: int = 0,
                           I: int = 0, out: Optional[torch.Tensor] = None,

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
         assert hasattr(lib, n), f"{n} declared in the header but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.omni_moe_abi_version() == _lib.ABI_VERSION == 5
+    assert lib.omni_moe_abi_version() == _lib.ABI_VERSION == 6
 
 
 def test_header_constants_match_binding():

@@ -1,0 +1,177 @@
+"""Router and layer in one library call against the router's call followed by the layer's: the same bits
+(output, routing weights, ids), on calls that route, quantise and sort in a single launch and on calls that do
+not fit that kernel."""
+import pytest
+import torch
+
+from tests.helpers import Layer, gen, tokens
+
+pytestmark = pytest.mark.gpu
+
+
+def _route_args(E, mode):
+    from omni_infer_amd import _lib as L
+    if mode == "noaux_tc":      # sigmoid + bias, groups by the sum of their two best (layer.py:341-351)
+        return dict(top_k=8, n_group=8, topk_group=4, score_fn="sigmoid", group_mode=L.OMNI_GROUP_TOP2SUM,
+                    masked_fill_zero=False, weight_from_c=False, renorm=True, scale=2.5, eps=1e-20)
+    if mode == "softmax":       # fused_topk (fused_moe.py:24-34)
+        return dict(top_k=2, n_group=1, topk_group=1, score_fn="softmax", group_mode=L.OMNI_GROUP_MAX,
+                    masked_fill_zero=False, weight_from_c=False, renorm=True, scale=1.0, eps=0.0)
+    raise AssertionError(mode)
+
+
+def _both(x, logits, bias, ra, lo, n, d, shared, H, I, rows_dtype=torch.float32, x_scale=None):
+    from omni_infer_amd import hip_ops as ops
+    w, ids = ops.moe_route(logits, bias, **ra)
+    want = ops.moe_w8a8_layer(x, x_scale, w, ids, lo, lo + n, d["w13"], d["s13"], d["w2"], d["s2"], shared, H=H, I=I,
+                              rows_dtype=rows_dtype)
+    got, gw, gids = ops.moe_w8a8_layer_routed(x, x_scale, logits, bias, lo=lo, hi=lo + n, w13_packed=d["w13"],
+                                              w13_scale=d["s13"], w2_packed=d["w2"], w2_scale=d["s2"], shared=shared,
+                                              H=H, I=I, rows_dtype=rows_dtype, **ra)
+    torch.cuda.synchronize()
+    return (want, w, ids), (got, gw, gids)
+
+
+def _same(a, b, what):
+    for u, v, name in zip(a, b, ("output", "routing weights", "ids")):
+        assert torch.equal(u, v), f"{what}: {name} differ"
+
+
+@pytest.mark.parametrize("T", [1, 3, 64, 130, 512])
+def test_single_launch_front_matches_two_calls(T):
+    """E=256 in 8 groups, top 8 of the 4 best groups, 32 local experts from id 64: the decode-sized calls whose
+    first launch routes, quantises and sorts.  Token counts that are not multiples of four leave routing
+    wavefronts without a token; every call reuses an arrival counter that an earlier call left behind."""
+    E, n, H, I, lo = 256, 32, 1024, 256, 64
+    lay = Layer(n, H, I, seed=401, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(402 + T)
+    ra = _route_args(E, "noaux_tc")
+    for rep in range(3):
+        x = tokens(T, H, 403 + rep).cuda()
+        logits = torch.randn(T, E, generator=g).cuda()
+        bias = (torch.randn(E, generator=g) * 0.1).cuda()
+        a, b = _both(x, logits, bias, ra, lo, n, d, shared, H, I)
+        _same(a, b, f"T={T} call {rep}")
+        assert bool(((a[2] >= lo) & (a[2] < lo + n)).any()) or T < 3
+
+
+def test_many_calls_in_a_row_reuse_the_counters():
+    """More calls than the library holds arrival counters: each counter is used again and must have been left
+    at zero by the call that used it before."""
+    E, n, H, I = 8, 8, 1024, 512
+    lay = Layer(n, H, I, seed=411, shared=False)
+    d = lay.to_device()
+    g = gen(412)
+    ra = _route_args(E, "softmax")
+    T = 37
+    x = tokens(T, H, 413).cuda()
+    logits = torch.randn(T, E, generator=g).cuda()
+    a, b = _both(x, logits, None, ra, 0, n, d, None, H, I)
+    _same(a, b, "first call")
+    from omni_infer_amd import hip_ops as ops
+    out = torch.empty_like(a[0])
+    for i in range(600):
+        ops.moe_w8a8_layer_routed(x, None, logits, None, lo=0, hi=n, w13_packed=d["w13"], w13_scale=d["s13"],
+                                  w2_packed=d["w2"], w2_scale=d["s2"], shared=None, H=H, I=I, out=out, **ra)
+        if i % 97 == 0:
+            torch.cuda.synchronize()
+            assert torch.equal(out, a[0]), f"call {i}"
+            out.zero_()
+    torch.cuda.synchronize()
+    assert torch.equal(out, a[0])
+
+
+@pytest.mark.parametrize("case", ["many_tokens", "int8_tokens", "bf16_rows"])
+def test_calls_outside_the_single_launch_front(case):
+    """More than 4096 assignments, or tokens that arrive quantised: the router runs as a launch of its own and the
+    results are still those of the two calls."""
+    E, n, H, I, lo = 64, 16, 512, 256, 8
+    lay = Layer(n, H, I, seed=421, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(422)
+    ra = _route_args(E, "noaux_tc")
+    T = 700 if case == "many_tokens" else 48
+    x = tokens(T, H, 423).cuda()
+    logits = torch.randn(T, E, generator=g).cuda()
+    bias = (torch.randn(E, generator=g) * 0.1).cuda()
+    xs = None
+    if case == "int8_tokens":
+        from omni_infer_amd import hip_ops as ops
+        x, xs = ops.npu_dynamic_quant(x)
+    rows_dtype = torch.bfloat16 if case == "bf16_rows" else torch.float32
+    a, b = _both(x, logits, bias, ra, lo, n, d, shared, H, I, rows_dtype=rows_dtype, x_scale=xs)
+    _same(a, b, case)
+
+
+def test_routed_entry_rejects_bad_routing_arguments():
+    from omni_infer_amd import hip_ops as ops
+    E, n, H, I = 64, 16, 512, 256
+    lay = Layer(n, H, I, seed=431, shared=False)
+    d = lay.to_device()
+    x = tokens(8, H, 432).cuda()
+    logits = torch.zeros(8, E, device="cuda")
+    ra = _route_args(E, "noaux_tc")
+    ra["n_group"] = 7   # does not divide 64
+    with pytest.raises(RuntimeError, match="n_group"):
+        ops.moe_w8a8_layer_routed(x, None, logits, None, lo=0, hi=n, w13_packed=d["w13"], w13_scale=d["s13"],
+                                  w2_packed=d["w2"], w2_scale=d["s2"], shared=None, H=H, I=I, **ra)
+    with pytest.raises(ValueError, match="one row of logits per token"):
+        ops.moe_w8a8_layer_routed(x, None, logits[:4], None, lo=0, hi=n, w13_packed=d["w13"], w13_scale=d["s13"],
+                                  w2_packed=d["w2"], w2_scale=d["s2"], shared=None, H=H, I=I,
+                                  **_route_args(E, "noaux_tc"))
+
+
+def test_routed_call_is_graph_capturable():
+    """The routed entry captured in a HIP graph and replayed with eager work in between: the arrival counter a
+    capture took is left at zero by every replay."""
+    E, n, H, I, K, T = 32, 4, 1024, 512, 8, 64
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+    lay = Layer(n, H, I, seed=441, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(442)
+    x = tokens(T, H, 443).cuda()
+    logits = torch.randn(T, E, generator=g).cuda()
+    bias = (torch.randn(E, generator=g) * 0.01).cuda()
+    ra = _route_args(E, "noaux_tc")
+    need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n, H, I, 1, L.OMNI_DT_F32)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out = torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
+    tw = torch.empty(T, K, dtype=torch.float32, device="cuda")
+    ti = torch.empty(T, K, dtype=torch.int32, device="cuda")
+
+    def step():
+        return ops.moe_w8a8_layer_routed(x, None, logits, bias, lo=0, hi=n, w13_packed=d["w13"], w13_scale=d["s13"],
+                                         w2_packed=d["w2"], w2_scale=d["s2"], shared=shared, H=H, I=I, workspace=ws,
+                                         out=out, topk_w=tw, topk_ids=ti, **ra)[0]
+
+    eager = step().clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        out.zero_()
+        ti.zero_()
+        junk = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager run"
+        del junk
+    x.copy_(tokens(T, H, 444).cuda())
+    logits.copy_(torch.randn(T, E, generator=g).cuda())
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = out.clone()
+    assert torch.equal(step(), replayed), "replay on new inputs differs from the eager run"
