@@ -695,6 +695,116 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
   }
 }
 
+// ---- which tile a block id names (shared by the tile kernels)
+// Real tiles (row blocks that exist x column tiles) get the ids [0, n_real): first the tiles of the heavy row
+// blocks, then those of the light ones; the last `left` real tiles (a last partial round of at most half the
+// chip) are each split `split` ways along the reduction, the helper shares have the ids [n_real, total).
+struct TileCount { int n_heavy, n_real, left, split, total; };
+struct TileSel { int bx, by, share, tail_tile; bool light; };
+constexpr int TILE_LIGHT_MAX = 96;
+
+template <bool LINES>
+__device__ __forceinline__ TileCount tile_count(const GemmArgs& a, int total_h, int total_l, int nk_all) {
+  TileCount t;
+  t.n_heavy = total_h * a.tile_gx;
+  t.n_real = (total_h + total_l) * a.tile_gx;
+  t.left = 0;
+  t.split = 1;
+  if (a.tail_part != nullptr && a.tile_slots > 0) {
+    t.left = t.n_real % a.tile_slots;
+    if (t.left > 0 && 2 * t.left <= a.tile_slots)
+      t.split = min(min(a.tile_split_max, a.tile_slots / t.left), LINES ? nk_all / 2 : nk_all);
+    if (t.split < 2) { t.split = 1; t.left = 0; }
+  }
+  t.total = t.n_real + t.left * (t.split - 1);
+  return t;
+}
+
+// false: the id names no work
+__device__ __forceinline__ bool tile_select(const GemmArgs& a, const TileCount& tc, int total_h, int total_l, int id,
+                                            TileSel& s) {
+  constexpr int TILE_PR = 4;
+  const int gx = a.tile_gx, pc = a.tile_pc, npc = gx / pc, per_patch = TILE_PR * pc;
+  s.share = 0;
+  s.tail_tile = -1;
+  if (id >= tc.n_real) {
+    const int h = id - tc.n_real;
+    if (tc.split == 1 || h >= tc.left * (tc.split - 1)) return false;
+    s.tail_tile = h / (tc.split - 1);
+    s.share = 1 + h % (tc.split - 1);
+    id = tc.n_real - tc.left + s.tail_tile;
+  } else if (tc.split > 1 && id >= tc.n_real - tc.left) {
+    s.tail_tile = id - (tc.n_real - tc.left);
+  }
+  s.light = id >= tc.n_heavy;
+  const int t = s.light ? id - tc.n_heavy : id;   // id inside the set
+  const int RB = s.light ? total_l : total_h;     // row blocks of the set
+  const int bulk_rows = RB / TILE_PR * TILE_PR;
+  const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
+  const int nA = patches8 * per_patch, nB = (patches - patches8) * per_patch;
+  if (t < nA + nB) {
+    int patch, q;
+    if (t < nA) {
+      // the tiles of a patch are 8 ids apart: one XCD runs them all
+      const int j = t >> 3;
+      patch = (j / per_patch) * 8 + (t & 7);
+      q = j % per_patch;
+    } else {
+      patch = patches8 + (t - nA) / per_patch;
+      q = (t - nA) % per_patch;
+    }
+    s.by = (patch / npc) * TILE_PR + q / pc;
+    s.bx = (patch % npc) * pc + q % pc;
+  } else {
+    s.by = bulk_rows + (t - nA - nB) / gx;
+    s.bx = (t - nA - nB) % gx;
+  }
+  return true;
+}
+
+// Hand-over between the shares of a split tile (their blocks may run on different XCDs, each with its own
+// L2).  Every wavefront stores its partial sums, all wavefronts meet at the block barrier, then one
+// thread counts in with a device-scope acquire-release add: the release half makes every store
+// that happened before it (the barrier orders the other wavefronts' stores before it) visible to
+// the device before the counter moves, and whoever reads the final count has, through the acquire
+// half and the chain of adds on the same counter, all other shares' stores visible to its block
+// after the second barrier.  No share ever waits for another.  True for the share that arrived last: its
+// accumulators then hold the sums of all shares.
+template <int WN>
+__device__ __forceinline__ bool tile_tail_handover(const GemmArgs& a, v16i (&acc)[4][2], int mt_count, int tail_tile,
+                                                   int split, int share, int w, int lane, int* s_last) {
+  constexpr int WAVE_INTS = 8 * 16 * WAVE;           // accumulator words of one wavefront
+  constexpr int TILE_INTS = 2 * WN * WAVE_INTS;
+  int32_t* mine = a.tail_part + ((size_t)tail_tile * split + share) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+    if (mt < mt_count) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine[((mt * 2 + t) * 16 + i) * WAVE] = acc[mt][t][i];
+    }
+  __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
+  __syncthreads();
+  if (threadIdx.x == 0)
+    *s_last = (__hip_atomic_fetch_add(a.tail_cnt + tail_tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == split - 1);
+  __syncthreads();
+  if (!*s_last) return false;
+  for (int s2 = 0; s2 < split; ++s2) {
+    if (s2 == share) continue;
+    const int32_t* theirs = a.tail_part + ((size_t)tail_tile * split + s2) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+      if (mt < mt_count) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mt][t][i] += theirs[((mt * 2 + t) * 16 + i) * WAVE];
+      }
+  }
+  return true;
+}
+
 // WN = 2: 256 threads, tile 256 x 128, two blocks per CU.  WN = 4: 512 threads, tile 256 x 256, one block
 // per CU (a third fewer operand bytes through the vector memory path per MFMA).
 // BF (GEMM1 only): round gate, up and their product to bf16 (the numerics of the reference's
@@ -740,56 +850,14 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // others.  Every share stores its int32 partial accumulators; whoever arrives last at the tile's
   // counter adds the others' to its own (integer sums: the order cannot matter) and runs the
   // epilogue.  Nobody waits for anybody.
-  constexpr int TILE_PR = 4;
-  constexpr int LIGHT_MAX = 96;
+  constexpr int LIGHT_MAX = TILE_LIGHT_MAX;
   const RowBlockKinds scan = row_block_kinds_scan(a.offsets, a.G, a.extra_rows, BM, LIGHT_MAX);
   const int nk_all = a.Kdim / 64;
-  int bx, by, split = 1, share = 0, tail_tile = -1;
-  bool light;
-  {
-    const int gx = a.tile_gx, pc = a.tile_pc, npc = gx / pc, per_patch = TILE_PR * pc;
-    const int n_heavy = scan.total_h * gx;
-    const int n_real = (scan.total_h + scan.total_l) * gx;
-    int left = 0;
-    if (a.tail_part != nullptr && a.tile_slots > 0) {
-      left = n_real % a.tile_slots;
-      if (left > 0 && 2 * left <= a.tile_slots) split = min(min(a.tile_split_max, a.tile_slots / left), LINES ? nk_all / 2 : nk_all);
-      if (split < 2) { split = 1; left = 0; }
-    }
-    int id = (int)blockIdx.x;
-    if (id >= n_real) {
-      const int h = id - n_real;
-      if (split == 1 || h >= left * (split - 1)) return;
-      tail_tile = h / (split - 1);
-      share = 1 + h % (split - 1);
-      id = n_real - left + tail_tile;
-    } else if (split > 1 && id >= n_real - left) {
-      tail_tile = id - (n_real - left);
-    }
-    light = id >= n_heavy;
-    const int t = light ? id - n_heavy : id;              // id inside the set
-    const int RB = light ? scan.total_l : scan.total_h;   // row blocks of the set
-    const int bulk_rows = RB / TILE_PR * TILE_PR;
-    const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
-    const int nA = patches8 * per_patch, nB = (patches - patches8) * per_patch;
-    if (t < nA + nB) {
-      int patch, q;
-      if (t < nA) {
-        // the tiles of a patch are 8 ids apart: one XCD runs them all
-        const int j = t >> 3;
-        patch = (j / per_patch) * 8 + (t & 7);
-        q = j % per_patch;
-      } else {
-        patch = patches8 + (t - nA) / per_patch;
-        q = (t - nA) % per_patch;
-      }
-      by = (patch / npc) * TILE_PR + q / pc;
-      bx = (patch % npc) * pc + q % pc;
-    } else {
-      by = bulk_rows + (t - nA - nB) / gx;
-      bx = (t - nA - nB) % gx;
-    }
-  }
+  const TileCount tc = tile_count<LINES>(a, scan.total_h, scan.total_l, nk_all);
+  TileSel sel;
+  if (!tile_select(a, tc, scan.total_h, scan.total_l, (int)blockIdx.x, sel)) return;
+  const int bx = sel.bx, by = sel.by, split = tc.split, share = sel.share, tail_tile = sel.tail_tile;
+  const bool light = sel.light;
   RowBlock rb;
   row_block_kinds_find(scan, a.offsets, a.G, a.extra_rows, BM, LIGHT_MAX, light, by, rb);
   // this block's k-steps [k_first, k_first + nk64)
@@ -937,42 +1005,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   if (tail_tile >= 0) {
     // one share of a split tile: publish the partial sums, count in, and only the last one goes on
     __shared__ int s_last;
-    constexpr int WAVE_INTS = 8 * 16 * WAVE;           // accumulator words of one wavefront
-    constexpr int TILE_INTS = 2 * WN * WAVE_INTS;
-    // Hand-over between the shares of a tile (their blocks may run on different XCDs, each with its own
-    // L2).  Every wavefront stores its partial sums, all wavefronts meet at the block barrier, then one
-    // thread counts in with a device-scope acquire-release add: the release half makes every store
-    // that happened before it (the barrier orders the other wavefronts' stores before it) visible to
-    // the device before the counter moves, and whoever reads the final count has, through the acquire
-    // half and the chain of adds on the same counter, all other shares' stores visible to its block
-    // after the second barrier.  No share ever waits for another.
-    int32_t* mine = a.tail_part + ((size_t)tail_tile * split + share) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-      if (mt < c.mt_count) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) mine[((mt * 2 + t) * 16 + i) * WAVE] = acc[mt][t][i];
-      }
-    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
-    __syncthreads();
-    if (threadIdx.x == 0)
-      s_last = (__hip_atomic_fetch_add(a.tail_cnt + tail_tile, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == split - 1);
-    __syncthreads();
-    if (!s_last) return;
-    for (int s2 = 0; s2 < split; ++s2) {
-      if (s2 == share) continue;
-      const int32_t* theirs = a.tail_part + ((size_t)tail_tile * split + s2) * TILE_INTS + (size_t)w * WAVE_INTS + lane;
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-        if (mt < c.mt_count) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[mt][t][i] += theirs[((mt * 2 + t) * 16 + i) * WAVE];
-        }
-    }
+    if (!tile_tail_handover<WN>(a, acc, c.mt_count, tail_tile, split, share, w, lane, &s_last)) return;
   }
   uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
   tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wm, wn, bx, row0, nrows, wsc, I);
