@@ -572,8 +572,8 @@ constexpr int TILE_OUT_PITCH_DW = 48;
 #define TILE_STAGE_DWORDS (32 * TILE_OUT_PITCH_DW)  // staging dwords of one wavefront
 template <int KIND, int WN, bool BF>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][2], const float* row_scale,
-                                              uint32_t* stage32, int lane, int wm, int wn, int bx, int row0,
-                                              int nrows, const float* __restrict__ wsc, int I) {
+                                              uint32_t* stage32, int lane, int wave_row0, int mt_count, int wn, int bx,
+                                              int row0, int nrows, const float* __restrict__ wsc, int I) {
   constexpr int NBS = 4 * WN;
   constexpr int GS = 2 * WN;
   // ---- epilogue, one 32-row tile at a time
@@ -602,8 +602,8 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
       uint32_t* const stage_lane = stage32 + (4 * (lane >> 5) + odd) * OUT_PITCH_DW + (c32 >> 1);
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) {
-        const int tile_r0 = wm * 128 + mt * 32;
-        if (tile_r0 < nrows) {
+        const int tile_r0 = wave_row0 + mt * 32;
+        if (mt < mt_count) {
           // accumulator entries i, i+1 (i even) are rows r, r+1 of the same channel; neighbouring
           // lanes hold neighbouring channels.  One pack, one lane exchange and one byte permute give
           // every lane a dword of two neighbouring channels: even lanes for row r, odd lanes for row r+1.
@@ -674,9 +674,10 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
     };
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
-      const int tile_r0 = wm * 128 + mt * 32;
+      const int tile_r0 = wave_row0 + mt * 32;
+      if (mt >= mt_count) continue;
       if (tile_r0 + 32 <= nrows) rows32(mt, tile_r0, std::true_type{});
-      else if (tile_r0 < nrows) rows32(mt, tile_r0, std::false_type{});
+      else rows32(mt, tile_r0, std::false_type{});
     }
   }
   // raw accumulators for the parity tests, kept out of the loops above so that none of their
@@ -686,8 +687,8 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int rr = wm * 128 + mt * 32 + tile32_row(lane, i);
-        if (rr < nrows) {
+        const int rr = wave_row0 + mt * 32 + tile32_row(lane, i);
+        if (mt < mt_count && rr < nrows) {
 #pragma unroll
           for (int t = 0; t < 2; ++t) a.acc_dbg[(size_t)(row0 + rr) * (size_t)a.N + ncol[t]] = acc[mt][t][i];
         }
@@ -886,7 +887,13 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   if constexpr (KIND == 1) { tile_strip0[0] = 2 * wn; tile_strip0[1] = GS + 2 * wn; }
   else { tile_strip0[0] = 4 * wn; tile_strip0[1] = 4 * wn + 2; }
   // 32-row tiles of this wavefront that hold rows of the block
-  c.mt_count = min(4, max(0, (nrows - wm * 128 + 31) / 32));
+  // The two wavefront rows of the block share its rows: in the 16x16x64 loop the second one starts at the first
+  // multiple of 32 past half the rows the block has (128 in a full block), so a block of 144 rows is 3 + 2
+  // row tiles of 32 and not 4 + 1: every k-step ends at a block barrier and takes as long as the wavefront with
+  // the most row tiles.  The other loops keep the fixed halves of 128.
+  const int half_rows = (LINES && M16) ? min(128, ((nrows + 1) / 2 + 31) / 32 * 32) : 128;
+  const int wave_row0 = wm * half_rows;
+  c.mt_count = (wm == 0) ? min(half_rows / 32, (nrows + 31) / 32) : min(4, max(0, (nrows - half_rows + 31) / 32));
   LineCtx lc;
   if constexpr (LINES) {
     lc.w = w;
@@ -926,7 +933,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
 #pragma unroll
       for (int e = 0; e < 2; ++e)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) lc.a16_off[e][h] = (wm * 128 + h * 16 + r16) * 8 + ((4 * e + (lane >> 4)) ^ swz);
+        for (int h = 0; h < 2; ++h) lc.a16_off[e][h] = (wave_row0 + h * 16 + r16) * 8 + ((4 * e + (lane >> 4)) ^ swz);
 #pragma unroll
       for (int n = 0; n < 4; ++n) lc.b16_off[n] = (tile_strip0[n >> 1] + (n & 1)) * WAVE + lane;
     }
@@ -1008,7 +1015,7 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     if (!tile_tail_handover<WN>(a, acc, c.mt_count, tail_tile, split, share, w, lane, &s_last)) return;
   }
   uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
-  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wm, wn, bx, row0, nrows, wsc, I);
+  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wave_row0, c.mt_count, wn, bx, row0, nrows, wsc, I);
 #endif
 }
 
