@@ -33,6 +33,9 @@ struct CombineArgs {
   const uint16_t* init;
   const void* post_add;
   const int32_t* post_add_row0;
+  // the added rows are bf16 rows of H values packed from row *post_add_row0 of an fp32 row buffer on (what
+  // GEMM2 writes for the extra group when the whole-layer entry asks for it); rows_dtype is fp32 then
+  int post_add_bf16;
   uint16_t* out;
 };
 
@@ -113,7 +116,24 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
     }
     // the row added after the rounding is requested with the first batch
     float pv[VEC];
-    if (a.post_add) load_vec<DT, false, VEC>(a.post_add, post_row, a.H, c, ncol, vec, pv);
+    if (a.post_add) {
+      if (DT == OMNI_DT_F32 && a.post_add_bf16) {
+        // bf16 row n of the packed rows begins 2 * row0 + n rows of H bf16 values into the buffer
+        const uint16_t* p = (const uint16_t*)a.post_add + (post_row + (size_t)*a.post_add_row0) * a.H + c;
+        if (ncol == VEC && vec) {
+          const v2i t = *(const v2i*)p;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            pv[2 * j] = bf16_to_f32((uint16_t)((uint32_t)t[j] & 0xffffu));
+            pv[2 * j + 1] = bf16_to_f32((uint16_t)((uint32_t)t[j] >> 16));
+          }
+        } else {
+          for (int j = 0; j < VEC; ++j) pv[j] = j < ncol ? bf16_to_f32(p[j]) : 0.0f;
+        }
+      } else {
+        load_vec<DT, false, VEC>(a.post_add, post_row, a.H, c, ncol, vec, pv);
+      }
+    }
     // eight rows are requested together, then added in list order (one multiply, one add per row)
     for (int j0 = 0; j0 < cnt; j0 += 8) {
       float v[8][VEC];
@@ -159,9 +179,10 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a) {
 
 }  // namespace
 
-extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* topk_w, const int32_t* src_to_dst,
-                                int idx_mode, int order, int T, int K, int H, const void* init_bf16,
-                                const void* post_add, const int32_t* post_add_row0, void* out_bf16, void* stream) {
+namespace {
+int combine_impl(const void* rows, int rows_dtype, const float* topk_w, const int32_t* src_to_dst, int idx_mode,
+                 int order, int T, int K, int H, const void* init_bf16, const void* post_add,
+                 const int32_t* post_add_row0, int post_add_bf16, void* out_bf16, void* stream) {
   if (T < 0 || K <= 0 || H <= 0) OMNI_FAIL(OMNI_E_INVALID, "combine: bad sizes T=%d K=%d H=%d", T, K, H);
   if (T == 0) return OMNI_OK;
   if (K > KMAX) OMNI_FAIL(OMNI_E_UNSUPPORTED, "combine: K=%d > %d", K, KMAX);
@@ -172,8 +193,10 @@ extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* t
   const uintptr_t out_align = (rows_dtype == OMNI_DT_BF16) ? 16 : 8;
   if (((uintptr_t)rows % 16) || ((uintptr_t)out_bf16 % out_align) || ((uintptr_t)post_add % 16))
     OMNI_FAIL(OMNI_E_INVALID, "combine: misaligned pointer");
+  if (post_add_bf16 && (rows_dtype != OMNI_DT_F32 || !post_add || !post_add_row0))
+    OMNI_FAIL(OMNI_E_INVALID, "combine: packed bf16 rows need fp32 rows and the extra group's first row");
   CombineArgs a{rows, rows_dtype, topk_w, src_to_dst, idx_mode, order, T, K, H, (const uint16_t*)init_bf16, post_add,
-                post_add_row0, (uint16_t*)out_bf16};
+                post_add_row0, post_add_bf16, (uint16_t*)out_bf16};
   // few tokens: one block per (token, chunk of 256 x 16 bytes) for parallelism; many tokens: one block
   // per token walks all chunks, so that a row's bytes are requested close together in time
   const int chunk_cols = 256 * ((rows_dtype == OMNI_DT_BF16) ? 8 : 4);
@@ -184,6 +207,14 @@ extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* t
   else hipLaunchKernelGGL(combine_kernel<OMNI_DT_BF16>, grid, block, 0, st, a);
   OMNI_CHECK_LAUNCH("combine");
   return OMNI_OK;
+}
+}  // namespace
+
+extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* topk_w, const int32_t* src_to_dst,
+                                int idx_mode, int order, int T, int K, int H, const void* init_bf16,
+                                const void* post_add, const int32_t* post_add_row0, void* out_bf16, void* stream) {
+  return combine_impl(rows, rows_dtype, topk_w, src_to_dst, idx_mode, order, T, K, H, init_bf16, post_add, post_add_row0,
+                      0, out_bf16, stream);
 }
 
 // ---------------------------------------------------------------- whole layer
@@ -308,15 +339,22 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
                                     sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),
                                     (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, tail != nullptr, stream);
   if (rc) return rc;
+  // The weighted sum rounds the shared expert's row to bf16 before it adds it to the rounded sum of the routed rows,
+  // so with fp32 rows GEMM2 writes that group's rows as bf16 straight away (into the first half of the space their
+  // fp32 form would take): the same bits, half the bytes written and read.  Only where GEMM2 runs the tile kernel,
+  // whose epilogue stores whole lines either way; the streaming kernel stores an element per lane, and 2-byte
+  // elements cost its few shared rows more than their bytes save (measured at 64 tokens: +0.5 us).
+  const bool shared_rows_bf16 = with_shared && L.rows_dtype == OMNI_DT_F32 && tail != nullptr;
   // GEMM1's scratch is free again once its row quantiser has run: GEMM2 takes it over (with cleared counters: the
   // split-tile scratch of GEMM1, whose counter words for GEMM2 nobody has touched since the sorting kernel)
   rc = omni_gemm2_dequant_impl((const int8_t*)(ws + L.h_q), (const float*)(ws + L.h_s), w2_packed, w2_scale, sh2_packed,
                                sh2_scale, extra, offsets, G, H, I, L.M_cap, L.rows_dtype, ws + L.rows, nullptr,
-                               tail ? tail : (void*)(ws + L.g1_ws), tail ? tail_bytes : L.g1_bytes, tail != nullptr, stream);
+                               tail ? tail : (void*)(ws + L.g1_ws), tail ? tail_bytes : L.g1_bytes, tail != nullptr,
+                               shared_rows_bf16, stream);
   if (rc) return rc;
-  return omni_moe_combine(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
-                          nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr, out_bf16,
-                          stream);
+  return combine_impl(ws + L.rows, L.rows_dtype, topk_w, src_to_dst, OMNI_IDX_TOKEN_MAJOR, OMNI_ORDER_SLOT, T, K, H,
+                      nullptr, with_shared ? ws + L.rows : nullptr, with_shared ? offsets + G : nullptr,
+                      shared_rows_bf16 ? 1 : 0, out_bf16, stream);
 }
 }  // namespace
 

@@ -70,7 +70,7 @@ int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const 
 int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
                             const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows, const int32_t* offsets,
                             int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out, int32_t* acc_dbg,
-                            void* workspace, size_t ws_bytes, bool counters_clean, void* stream);
+                            void* workspace, size_t ws_bytes, bool counters_clean, bool extra_rows_bf16, void* stream);
 
 // ---------------------------------------------------------------- specified transcendental
 // exp with a fixed operation sequence: clamp to [-87, 87], Cody-Waite reduction by ln2 split in

@@ -573,13 +573,16 @@ constexpr int TILE_OUT_PITCH_DW = 48;
 template <int KIND, int WN, bool BF>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][2], const float* row_scale,
                                               uint32_t* stage32, int lane, int wave_row0, int mt_count, int wn, int bx,
-                                              int row0, int nrows, const float* __restrict__ wsc, int I) {
+                                              int row0, int nrows, const float* __restrict__ wsc, int I,
+                                              int bf16_shift) {
   constexpr int NBS = 4 * WN;
   constexpr int GS = 2 * WN;
   // ---- epilogue, one 32-row tile at a time
   const int c32 = lane & 31;
   constexpr int OUT_PITCH_DW = TILE_OUT_PITCH_DW;
-  const bool bf16_out = (KIND == 2) && a.out_dtype == OMNI_DT_BF16;
+  // bf16_shift >= 0: bf16 rows of the extra group inside an fp32 row buffer (GemmArgs::extra_rows_bf16)
+  const bool bf16_out = (KIND == 2) && (a.out_dtype == OMNI_DT_BF16 || bf16_shift >= 0);
+  const int out_row0 = row0 + (bf16_shift >= 0 ? bf16_shift : 0);  // first row of the block in bf16 rows
   constexpr bool bf = BF;
   float wsc_g[2];
   int ncol[2];
@@ -629,7 +632,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
             const int rr = tile_r0 + r;
             v4i v = *(const v4i*)(stage32 + r * OUT_PITCH_DW + (lane & 7) * 4);
             if (rr < nrows)  // read once, by the combine
-              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
+              __builtin_nontemporal_store(v, (v4i*)((uint16_t*)a.rows_out + (size_t)(out_row0 + rr) * a.N + (ncol[0] - c32) + (lane & 7) * 8));
           }
           __builtin_amdgcn_wave_barrier();
         }
@@ -1015,7 +1018,12 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
     if (!tile_tail_handover<WN>(a, acc, c.mt_count, tail_tile, split, share, w, lane, &s_last)) return;
   }
   uint32_t* stage32 = (uint32_t*)(w < 2 ? sa0 : (w < 4 ? sa1 : (w < 6 ? sa2 : sb0))) + (w & 1) * TILE_STAGE_DWORDS;
-  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wave_row0, c.mt_count, wn, bx, row0, nrows, wsc, I);
+  int bf16_shift = -1;
+  if constexpr (KIND == 2) {
+    if (a.extra_rows_bf16 && a.out_dtype == OMNI_DT_F32 && g >= a.G) bf16_shift = a.offsets[a.G];
+  }
+  tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wave_row0, c.mt_count, wn, bx, row0, nrows, wsc, I,
+                              bf16_shift);
 #endif
 }
 
@@ -1442,13 +1450,13 @@ extern "C" int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, c
                                       int out_dtype, void* rows_out, int32_t* acc_dbg, void* workspace, size_t ws_bytes,
                                       void* stream) {
   return omni_gemm2_dequant_impl(h_q, h_scale, w2_packed, w2_scale, w2_extra, w2_extra_scale, extra_rows, offsets, G, H, I,
-                                 M_cap, out_dtype, rows_out, acc_dbg, workspace, ws_bytes, false, stream);
+                                 M_cap, out_dtype, rows_out, acc_dbg, workspace, ws_bytes, false, false, stream);
 }
 
 int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
                             const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows, const int32_t* offsets,
                             int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out, int32_t* acc_dbg,
-                            void* workspace, size_t ws_bytes, bool counters_clean, void* stream) {
+                            void* workspace, size_t ws_bytes, bool counters_clean, bool extra_rows_bf16, void* stream) {
   int rc = check_group_args("gemm2", offsets, G, H, I, M_cap, extra_rows, w2_extra, w2_extra_scale);
   if (rc) return rc;
   if (M_cap == 0) return OMNI_OK;
@@ -1463,6 +1471,9 @@ int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = I; a.N = H; a.flags = 0;
   a.rows_out = rows_out; a.out_dtype = out_dtype; a.acc_dbg = acc_dbg; a.S = 1; a.M_cap = M_cap;
   Plan p = make_plan<2>(a.T, a.K, G, extra_rows, I, H, M_cap);
+  if (extra_rows_bf16 && !(p.tile && out_dtype == OMNI_DT_F32 && extra_rows > 0))
+    OMNI_FAIL(OMNI_E_INVALID, "gemm2: packed bf16 rows of the extra group are written by the tile kernel into fp32 rows only");
+  a.extra_rows_bf16 = extra_rows_bf16 ? 1 : 0;
   if (workspace && ((uintptr_t)workspace % 256)) OMNI_FAIL(OMNI_E_INVALID, "gemm2: workspace must be 256-byte aligned");
   return dispatch_gemm<2>(a, p, M_cap, workspace, workspace ? ws_bytes : 0, counters_clean, (hipStream_t)stream, "gemm2");
 }

@@ -23,6 +23,10 @@ struct GemmArgs {
   float* y;            // GEMM1: [M_cap, I]
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
+  // Tile kernel, GEMM2 with fp32 rows: the extra group's rows are written as bf16 all the same, H bf16 values
+  // each, packed from where that group's fp32 rows would begin (the whole-layer entry asks for this: the weighted
+  // sum rounds the shared expert's rows to bf16 before it adds them, so the bits are the same and half the bytes move)
+  int extra_rows_bf16;
   int32_t* acc_dbg;    // [M_cap, N], nullable
   int tile_gx, tile_gy, tile_pc;  // tile kernel: column tiles, row blocks (worst case), columns of a patch
   int tile_slots;                 // tile kernel: blocks the chip runs at once
