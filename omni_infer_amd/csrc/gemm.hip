@@ -705,7 +705,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
 // chip) are each split `split` ways along the reduction, the helper shares have the ids [n_real, total).
 struct TileCount { int n_heavy, n_real, left, split, total; };
 struct TileSel { int bx, by, share, tail_tile; bool light; };
-constexpr int TILE_LIGHT_MAX = 96;
+[[maybe_unused]] constexpr int TILE_LIGHT_MAX = 96;
 
 template <bool LINES>
 __device__ __forceinline__ TileCount tile_count(const GemmArgs& a, int total_h, int total_l, int nk_all) {

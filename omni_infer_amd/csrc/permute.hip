@@ -6,8 +6,11 @@
 // chunk 64 assignments at a time, finds the lanes that hold the same bucket with one ballot per
 // bucket-id bit, and keeps a running per-bucket count in an LDS histogram (one per wavefront).
 // An exclusive prefix over wavefronts, blocks and buckets then gives every assignment its slot.
-// Small inputs (<= 4096 assignments) are sorted by one block in one launch; larger ones take a
-// count launch, a one-block scan launch and a scatter launch.
+// Small inputs (<= 4096 assignments) are sorted by one block in one launch: four wavefronts up to 1024
+// assignments (a block of four starts sooner than one of sixteen: measured better up to 128 tokens of 8), sixteen
+// wavefronts above; either way a wavefront has at most four dependent passes.  Larger inputs take a count launch,
+// a one-block scan launch and a scatter launch.
+#include <stdlib.h>
 #include <atomic>
 #include <mutex>
 #include "common.h"
@@ -20,6 +23,7 @@ constexpr int GMAX = 256;        // local experts per call
 constexpr int NB = GMAX + 1;     // buckets incl. the dropped one
 constexpr int CH_MULTI = 1024;   // assignments per block in the multi-block path
 constexpr int CH_SINGLE = 4096;  // largest input of the single-block path
+constexpr int NW_SMALL_MAX_N = 1024;  // up to this many assignments the single block has 4 wavefronts, above 16
 
 struct PermArgs {
   const int32_t* ids;
@@ -35,7 +39,7 @@ struct PermArgs {
 };
 
 __device__ __forceinline__ void clear_words(const PermArgs& a) {
-  for (int i = threadIdx.x; i < a.zero_n; i += 256) a.zero_words[i] = 0;
+  for (int i = threadIdx.x; i < a.zero_n; i += blockDim.x) a.zero_words[i] = 0;
 }
 
 __device__ __forceinline__ int bucket_of(int id, int lo, int G) {
@@ -58,11 +62,11 @@ __device__ __forceinline__ void load_buckets(const PermArgs& a, int base, int le
 
 // Ranks the chunk [base, base+len): lrank[i] = number of earlier assignments of the same bucket
 // inside the same wavefront's part; whist[w][b] = count of bucket b in wavefront w's part.
-template <int MP>
+template <int MP, int NW = 4>
 __device__ __forceinline__ void rank_chunk(const PermArgs& a, int len, int passes, int (*whist)[NB], int* lrank,
                                            const int (&bk)[MP]) {
   const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
-  for (int i = threadIdx.x; i < 4 * NB; i += 256) (&whist[0][0])[i] = 0;
+  for (int i = threadIdx.x; i < NW * NB; i += NW * WAVE) (&whist[0][0])[i] = 0;
   __syncthreads();
   const int nbits = 32 - __clz(a.G);
   const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -139,63 +143,149 @@ __device__ __forceinline__ void wave0_excl_scan(const int* tot, int* off, int nb
   }
 }
 
+// The whole sort by one block of NW wavefronts.  After the ranking a thread per bucket turns the
+// wavefronts' counts of its bucket into their exclusive prefix (and the bucket's total), so that an assignment's
+// slot is three LDS reads: the bucket's base, its wavefront's prefix, its rank inside the wavefront.
+template <int NW>
 __device__ __forceinline__ void permute_single_body(const PermArgs& a) {
-  __shared__ int whist[4][NB];
+  constexpr int NT = NW * WAVE, MP = (NW == 4 ? NW_SMALL_MAX_N : CH_SINGLE) / NT;  // passes of a wavefront at most
+  __shared__ int whist[NW][NB];
   __shared__ int lrank[CH_SINGLE];
   __shared__ int tot[NB];
   __shared__ int off[NB + 1];
-  const int passes = (a.n + 255) / 256;
-  int bk[CH_SINGLE / 256];
+  const int passes = (a.n + NT - 1) / NT;
+  int bk[MP];
   load_buckets(a, 0, a.n, passes, bk);
   clear_words(a);
-  rank_chunk(a, a.n, passes, whist, lrank, bk);
+  rank_chunk<MP, NW>(a, a.n, passes, whist, lrank, bk);
   const int nb = a.G + 1;
-  for (int b = threadIdx.x; b < nb; b += 256) tot[b] = whist[0][b] + whist[1][b] + whist[2][b] + whist[3][b];
+  for (int b = threadIdx.x; b < nb; b += NT) {
+    int c[NW];
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) c[ww] = whist[ww][b];
+    int run = 0;
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) {
+      whist[ww][b] = run;
+      run += c[ww];
+    }
+    tot[b] = run;
+  }
   __syncthreads();
   wave0_excl_scan(tot, off, nb);
   __syncthreads();
-  for (int b = threadIdx.x; b < a.G; b += 256) {
+  for (int b = threadIdx.x; b < a.G; b += NT) {
     a.counts[b] = tot[b];
     a.offsets[b] = off[b];
   }
   if (threadIdx.x == 0) a.offsets[a.G] = off[a.G];
-  scatter_chunk(a, 0, passes, whist, lrank, off, bk);
+  const int w = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int j = 0; j < MP; ++j) {
+    if (j >= passes) break;
+    const int i = (w * passes + j) * WAVE + lane;
+    if (bk[j] >= 0) {
+      const int b = bk[j];
+      const int slot = off[b] + whist[w][b] + lrank[i];
+      const int src = src_index(a, i);
+      a.sorted_src[slot] = src;
+      a.src_to_dst[src] = (b < a.G) ? slot : -1;
+    }
+  }
 }
 
-__global__ __launch_bounds__(256) void permute_single(PermArgs a) { permute_single_body(a); }
+template <int NW>
+__global__ __launch_bounds__(NW * WAVE) void permute_single(PermArgs a) { permute_single_body<NW>(a); }
 
-// One launch for the two independent first steps of a small layer call: blocks [0, rows) quantise
-// one bf16 token row each, the last block sorts the assignments.
+// NW / 4 token rows of a block of NW wavefronts, four wavefronts a row: the row body of quant_rows.h with the
+// block barrier shared by the rows (rows past the end take part in it and touch no memory).
 template <int MAXV>
-__global__ __launch_bounds__(256) void quant_permute_small(const void* __restrict__ x, int64_t rows, int cols,
-                                                           int8_t* __restrict__ q, float* __restrict__ scale,
-                                                           PermArgs a) {
-  __shared__ float red[4];
-  if ((int64_t)blockIdx.x < rows) quant_row_vec_body<OMNI_DT_BF16, MAXV>(x, (int64_t)blockIdx.x, cols, cols, q, scale, red);
-  else permute_single_body(a);
+__device__ __forceinline__ void quant_four_rows(const void* __restrict__ xv, int64_t r0, int64_t rows, int cols,
+                                                int8_t* __restrict__ q, float* __restrict__ scale, float* red) {
+  const int tid = threadIdx.x & 255, qd = threadIdx.x >> 8;
+  const int64_t r = r0 + qd;
+  const bool live = r < rows;
+  const uint16_t* x = (const uint16_t*)xv + (live ? r : 0) * (int64_t)cols;
+  const int nvec = cols / 8;
+  float v[MAXV][8];
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int vi = tid + i * 256;
+    if (live && vi < nvec) {
+      const v4i raw = __builtin_nontemporal_load((const v4i*)(x + (size_t)vi * 8));  // the row is read once here
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t u = (uint32_t)raw[j];
+        v[i][2 * j] = bf16_to_f32((uint16_t)(u & 0xffffu));
+        v[i][2 * j + 1] = bf16_to_f32((uint16_t)(u >> 16));
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+    }
+  }
+  amax = wave_allmax_f(amax);
+  if ((threadIdx.x & (WAVE - 1)) == 0) red[threadIdx.x / WAVE] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[4 * qd], red[4 * qd + 1]), fmaxf(red[4 * qd + 2], red[4 * qd + 3]));
+  if (!live) return;  // (a block of four wavefronts has one row, qd = 0)
+  const float s = amax / 127.0f;
+  if (tid == 0) scale[r] = s;
+  int8_t* qr = q + r * (int64_t)cols;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int vi = tid + i * 256;
+    if (vi < nvec) {
+      uint32_t w0 = 0, w1 = 0;
+      if (s > 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          w0 |= ((uint32_t)(quant_i8(v[i][j], s) & 0xff)) << (8 * j);
+          w1 |= ((uint32_t)(quant_i8(v[i][4 + j], s) & 0xff)) << (8 * j);
+        }
+      }
+      const v2i o = {(int)w0, (int)w1};
+      *(v2i*)(qr + (size_t)vi * 8) = o;
+    }
+  }
 }
 
-// One launch for the three first steps of a small layer call: blocks [0, ceil(T/4)) route four tokens each (one
-// per wavefront), the other T blocks quantise one bf16 token row each, and the routing block that finishes last
-// sorts the assignments.  `arrive` counts the routing blocks that are done.  It is zero when the kernel starts and
-// the sorting block sets it back to zero, so no launch ever has to clear it.  The hand-over is the one of the
-// split tiles of the grouped GEMM: every wavefront waits for its stores, the block meets at a barrier, one
-// thread counts in with a device-scope acquire-release add (the release half makes the block's stores visible to
-// the device, the acquire half of the last add makes everybody else's visible to the sorting block).  No block
-// waits for another.
-template <int MAXV, int V>
-__global__ __launch_bounds__(256) void route_quant_permute_small(const void* __restrict__ x, int64_t rows, int cols,
+// One launch for the two independent first steps of a small layer call: blocks [0, ceil(rows / (NW/4))) quantise
+// NW / 4 bf16 token rows each, the last block sorts the assignments.
+template <int MAXV, int NW>
+__global__ __launch_bounds__(NW * WAVE) void quant_permute_small(const void* __restrict__ x, int64_t rows, int cols,
                                                                  int8_t* __restrict__ q, float* __restrict__ scale,
-                                                                 RouteArgs r, PermArgs a, int* arrive) {
-  __shared__ float red[4];
+                                                                 PermArgs a) {
+  constexpr int RPB = NW / 4;
+  __shared__ float red[NW];
+  const int quant_blocks = (int)((rows + RPB - 1) / RPB);
+  if ((int)blockIdx.x < quant_blocks) quant_four_rows<MAXV>(x, (int64_t)blockIdx.x * RPB, rows, cols, q, scale, red);
+  else permute_single_body<NW>(a);
+}
+
+// One launch for the three first steps of a small layer call: blocks [0, ceil(T/NW)) route NW tokens each
+// (one per wavefront), the next ceil(T/(NW/4)) blocks quantise NW/4 bf16 token rows each, and the routing block that
+// finishes last sorts the assignments.  `arrive` counts the routing blocks that are done.  It is zero when the
+// kernel starts and the sorting block sets it back to zero, so no launch ever has to clear it.  The hand-over is
+// the one of the split tiles of the grouped GEMM: every wavefront waits for its stores, the block meets at a
+// barrier, one thread counts in with a device-scope acquire-release add (the release half makes the block's stores
+// visible to the device, the acquire half of the last add makes everybody else's visible to the sorting block).
+// No block waits for another.
+template <int MAXV, int V, int NW>
+__global__ __launch_bounds__(NW * WAVE) void route_quant_permute_small(const void* __restrict__ x, int64_t rows,
+                                                                       int cols, int8_t* __restrict__ q,
+                                                                       float* __restrict__ scale, RouteArgs r,
+                                                                       PermArgs a, int* arrive) {
+  constexpr int RPB = NW / 4;
+  __shared__ float red[NW];
   __shared__ int s_last;
-  const int route_blocks = (r.T + 3) / 4;
+  const int route_blocks = (r.T + NW - 1) / NW;
   if ((int)blockIdx.x >= route_blocks) {
-    quant_row_vec_body<OMNI_DT_BF16, MAXV>(x, (int64_t)blockIdx.x - route_blocks, cols, cols, q, scale, red);
+    quant_four_rows<MAXV>(x, ((int64_t)blockIdx.x - route_blocks) * RPB, rows, cols, q, scale, red);
     return;
   }
   const int lane = threadIdx.x & (WAVE - 1);
-  const int t = (int)blockIdx.x * 4 + threadIdx.x / WAVE;
+  const int t = (int)blockIdx.x * NW + threadIdx.x / WAVE;
   if (t < r.T) {  // the same for a whole wavefront
     float s[V], bias[V];
     bool in[V];
@@ -211,7 +301,7 @@ __global__ __launch_bounds__(256) void route_quant_permute_small(const void* __r
   }
   __syncthreads();
   if (!s_last) return;
-  permute_single_body(a);
+  permute_single_body<NW>(a);
 }
 
 __global__ __launch_bounds__(256) void permute_count(PermArgs a) {
@@ -303,6 +393,20 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(GatherArgs g) {
 
 }  // namespace
 
+namespace {
+// wavefronts of the block that sorts a small input (and of the launch it is part of); OMNI_MOE_SORT_WAVES = 4 or
+// 16 overrides the choice (a tuning aid, read once)
+int sort_waves(int n) {
+  static const int forced = [] {
+    const char* e = getenv("OMNI_MOE_SORT_WAVES");
+    const int v = e ? atoi(e) : 0;
+    return (v == 4 || v == 16) ? v : 0;
+  }();
+  if (n > NW_SMALL_MAX_N) return 16;  // four wavefronts hold no more
+  return forced ? forced : 4;
+}
+}  // namespace
+
 extern "C" size_t omni_moe_permute_workspace_bytes(int T, int K, int n_local) {
   (void)n_local;
   int64_t n = (int64_t)T * K;
@@ -334,7 +438,8 @@ int omni_moe_permute_clearing(const int32_t* topk_ids, int T, int K, int lo, int
   PermArgs a{topk_ids, n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, (int32_t*)workspace, 0,
              zero_words, zero_words ? zero_n : 0};
   if (n <= CH_SINGLE) {
-    hipLaunchKernelGGL(permute_single, dim3(1), dim3(256), 0, st, a);
+    if (sort_waves(n) == 4) hipLaunchKernelGGL(permute_single<4>, dim3(1), dim3(4 * WAVE), 0, st, a);
+    else hipLaunchKernelGGL(permute_single<16>, dim3(1), dim3(16 * WAVE), 0, st, a);
     OMNI_CHECK_LAUNCH("permute_single");
     return OMNI_OK;
   }
@@ -358,11 +463,21 @@ int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float*
   if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((size_t)H * 2) % 16 != 0) return 1;
   PermArgs a{topk_ids, (int)n, T, K, lo, G, idx_mode, sorted_src, src_to_dst, counts, offsets, nullptr, 0,
              zero_words, zero_words ? zero_n : 0};
-  dim3 grid((unsigned)T + 1), block(256);
+  const int nw = sort_waves((int)n), rpb = nw / 4;
+  dim3 grid((unsigned)((T + rpb - 1) / rpb + 1)), block(nw * WAVE);
   hipStream_t st = (hipStream_t)stream;
-  if (H <= 8 * 256 * 1) hipLaunchKernelGGL(quant_permute_small<1>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
-  else if (H <= 8 * 256 * 2) hipLaunchKernelGGL(quant_permute_small<2>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
-  else hipLaunchKernelGGL(quant_permute_small<4>, grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a);
+  const int MV = H <= 8 * 256 ? 1 : (H <= 8 * 256 * 2 ? 2 : 4);
+#define QP_LAUNCH(MAXV, NW_) hipLaunchKernelGGL((quant_permute_small<MAXV, NW_>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, a)
+#define QP_NW(MAXV)             \
+  do {                          \
+    if (nw == 4) QP_LAUNCH(MAXV, 4); \
+    else QP_LAUNCH(MAXV, 16);   \
+  } while (0)
+  if (MV == 1) QP_NW(1);
+  else if (MV == 2) QP_NW(2);
+  else QP_NW(4);
+#undef QP_NW
+#undef QP_LAUNCH
   OMNI_CHECK_LAUNCH("quant_permute");
   return OMNI_OK;
 }
@@ -419,12 +534,16 @@ int omni_route_quant_permute_fused(const OmniRouteParams* rp, const void* x_bf16
               rp->topk_ids};
   PermArgs a{rp->topk_ids, (int)n, T, K, lo, G, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, counts, offsets, nullptr, 0,
              zero_words, zero_words ? zero_n : 0};
-  dim3 grid((unsigned)(T + (T + 3) / 4)), block(256);
+  const int nw = sort_waves((int)n), rpb = nw / 4;
+  dim3 grid((unsigned)((T + nw - 1) / nw + (T + rpb - 1) / rpb)), block(nw * WAVE);
   hipStream_t st = (hipStream_t)stream;
   const int V = (rp->E + 63) / 64;
   const int MV = H <= 8 * 256 ? 1 : (H <= 8 * 256 * 2 ? 2 : 4);
-#define RQP_LAUNCH(MAXV, VV) \
-  hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, r, a, arrive)
+#define RQP_LAUNCH(MAXV, VV)                                                                                                  \
+  do {                                                                                                                        \
+    if (nw == 4) hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 4>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, r, a, arrive); \
+    else hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 16>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, r, a, arrive);       \
+  } while (0)
 #define RQP_V(MAXV)                      \
   do {                                   \
     if (V <= 1) RQP_LAUNCH(MAXV, 1);     \

@@ -111,7 +111,10 @@ def test_dynamic_quant_strided_and_3d(ops):
 # ------------------------------------------------------------------ permutation
 @pytest.mark.parametrize("T,K,E,lo,hi", [(64, 8, 256, 0, 32), (64, 8, 256, 96, 128), (1, 8, 256, 0, 32),
                                          (500, 8, 256, 32, 64), (2048, 8, 256, 0, 32), (700, 6, 64, 0, 64),
-                                         (64, 2, 8, 0, 8), (1100, 8, 256, 0, 256)])
+                                         (64, 2, 8, 0, 8), (1100, 8, 256, 0, 256),
+                                         # either side of the sizes where the sort changes its block shape
+                                         (100, 8, 256, 0, 32), (128, 8, 256, 0, 32), (129, 8, 256, 0, 32),
+                                         (512, 8, 256, 0, 32), (513, 8, 256, 0, 32)])
 def test_permute_v2(ops, T, K, E, lo, hi):
     g = gen(8)
     ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
