@@ -175,3 +175,35 @@ def test_routed_call_is_graph_capturable():
     torch.cuda.synchronize()
     replayed = out.clone()
     assert torch.equal(step(), replayed), "replay on new inputs differs from the eager run"
+
+
+@pytest.mark.parametrize("T", [300, 777])
+def test_layer_entry_matches_the_separate_operators_at_tile_sizes(T):
+    """The layer entry against quantise, sort, GEMM1, GEMM2 and weighted sum called one by one, where both grouped
+    GEMMs run the tile kernel: inside the entry the shared expert's rows go from GEMM2 to the weighted sum as bf16
+    (packed into the front half of their fp32 place), outside they stay fp32 and are rounded by the weighted sum;
+    the bits must be the same.  The token counts leave a last row block of 44 and of 9 shared rows."""
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+    H, I, n, E, K, lo = 1024, 512, 8, 16, 4, 3
+    lay = Layer(n, H, I, seed=451, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(452 + T)
+    x = tokens(T, H, 453).cuda()
+    ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32).cuda()
+    w = torch.rand(T, K, generator=g).cuda()
+    assert "gemm_pipe" in ops.gemm_kernel_name(2, T, K, n, T, T * K + T, H, I)
+    got = ops.moe_w8a8_layer(x, None, w, ids, lo, lo + n, d["w13"], d["s13"], d["w2"], d["s2"], shared, H=H, I=I)
+
+    xq, xs = ops.npu_dynamic_quant(x)
+    p = ops.moe_permute(ids, lo, lo + n, L.OMNI_IDX_TOKEN_MAJOR)
+    M_cap = T * K + T
+    hq, hs, _ = ops.grouped_gemm1_swiglu_quant(xq, xs, p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, d["w13"], d["s13"],
+                                               p.offsets, H, I, M_cap, extra=(d["sh13"], d["sh_s13"]), extra_rows=T)
+    rows, _ = ops.grouped_gemm2_dequant(hq, hs, d["w2"], d["s2"], p.offsets, H, I, out_dtype=torch.float32,
+                                        extra=(d["sh2"], d["sh_s2"]), extra_rows=T)
+    want = ops.moe_combine(rows, w, p.src_to_dst, L.OMNI_IDX_TOKEN_MAJOR, L.OMNI_ORDER_SLOT, post_add=rows,
+                           post_add_row0=p.offsets[n:])
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
