@@ -324,6 +324,11 @@ size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int
  * topk_ids [T,K] int32 are outputs here and hold the routing when the call's work is done, everything else is
  * as for omni_moe_w8a8_layer, workspace size included.  Small calls (bf16 tokens, T*K <= 4096, H <= 8192) route,
  * quantise and sort in a single launch; other calls run the router's own launch first.
+ *   The single launch counts its finished routing blocks in one of 256 arrival counters that the library keeps in
+ *   static device memory (1 KiB per GPU, zero when the library is loaded).  Calls take the counters in turn and
+ *   every launch leaves its counter at zero, so nothing is asked of the caller as long as fewer than 256 such
+ *   calls are in flight on one GPU at a time.  The first such call on a device looks up that device's copy of the
+ *   counters: make it outside a stream capture.
  */
 int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const float* x_scale_in, const float* logits,
                                const float* bias, int E, int n_group, int topk_group, int score_fn, int group_mode,
