@@ -207,3 +207,38 @@ def test_layer_entry_matches_the_separate_operators_at_tile_sizes(T):
                            post_add_row0=p.offsets[n:])
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+
+
+def test_routed_calls_on_two_streams_do_not_share_a_counter():
+    """Two streams, each with its own workspace and outputs, issue routed calls without waiting for each other: calls
+    in flight at the same time hold different arrival counters, so both streams get the bits of a call made alone."""
+    from omni_infer_amd import _lib as L
+    from omni_infer_amd import hip_ops as ops
+    E, n, H, I, K = 32, 4, 1024, 512, 8
+    lay = Layer(n, H, I, seed=461, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    ra = _route_args(E, "noaux_tc")
+    g = gen(462)
+    jobs = []
+    for T in (64, 47):
+        x = tokens(T, H, 463 + T).cuda()
+        logits = torch.randn(T, E, generator=g).cuda()
+        bias = (torch.randn(E, generator=g) * 0.01).cuda()
+        need = L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, n, H, I, 1, L.OMNI_DT_F32)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        out = torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
+        tw = torch.empty(T, K, dtype=torch.float32, device="cuda")
+        ti = torch.empty(T, K, dtype=torch.int32, device="cuda")
+        kw = dict(lo=0, hi=n, w13_packed=d["w13"], w13_scale=d["s13"], w2_packed=d["w2"], w2_scale=d["s2"], shared=shared,
+                  H=H, I=I, workspace=ws, out=out, topk_w=tw, topk_ids=ti, **ra)
+        alone = ops.moe_w8a8_layer_routed(x, None, logits, bias, **kw)[0].clone()
+        jobs.append((x, logits, bias, kw, out, alone, torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    for rep in range(40):
+        for x, logits, bias, kw, out, alone, stream in jobs:
+            with torch.cuda.stream(stream):
+                ops.moe_w8a8_layer_routed(x, None, logits, bias, **kw)
+    torch.cuda.synchronize()
+    for x, logits, bias, kw, out, alone, stream in jobs:
+        assert torch.equal(out, alone)
