@@ -339,11 +339,7 @@ struct RowBlockKinds {
 // and a few rows more: there the small block stays next to the full one, whose weight panel it shares (deferred
 // to the end it would fetch that panel a second time, and with one full block per group that doubles the traffic).
 __device__ __forceinline__ bool last_block_is_light(int c, int BM, int light_max) {
-#ifdef OMNI_PROBE_LIGHT_ALWAYS
-  return (c % BM) > 0 && (c % BM) <= light_max;
-#else
   return (c % BM) > 0 && (c % BM) <= light_max && c / BM != 1;
-#endif
 }
 __device__ __forceinline__ int heavy_blocks(int c, int BM, int light_max) {
   return c / BM + ((c % BM) > 0 && !last_block_is_light(c, BM, light_max));
