@@ -242,3 +242,48 @@ def test_routed_calls_on_two_streams_do_not_share_a_counter():
     torch.cuda.synchronize()
     for x, logits, bias, kw, out, alone, stream in jobs:
         assert torch.equal(out, alone)
+
+
+@pytest.mark.parametrize("E,n_group,topk_group,K", [(40, 1, 1, 4), (384, 8, 3, 6), (512, 4, 2, 8)])
+def test_single_launch_front_with_other_expert_counts(E, n_group, topk_group, K):
+    """Expert counts that give a lane 1, 6 and 8 experts (40 leaves lanes without an expert), with and without
+    groups; the local range lies where only part of the assignments fall into it."""
+    from omni_infer_amd import _lib as L
+    n, H, I, lo, T = 8, 512, 256, 16, 50
+    lay = Layer(n, H, I, seed=471, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(472 + E)
+    ra = dict(top_k=K, n_group=n_group, topk_group=topk_group, score_fn="sigmoid", group_mode=L.OMNI_GROUP_TOP2SUM,
+              masked_fill_zero=False, weight_from_c=False, renorm=True, scale=2.5, eps=1e-20)
+    x = tokens(T, H, 473).cuda()
+    logits = torch.randn(T, E, generator=g).cuda()
+    bias = (torch.randn(E, generator=g) * 0.1).cuda()
+    a, b = _both(x, logits, bias, ra, lo, n, d, shared, H, I)
+    _same(a, b, f"E={E}")
+
+
+def test_routed_entry_when_nothing_is_local_and_when_there_are_no_tokens():
+    """No assignment falls into the local range: the output is the shared expert's alone (and zero without one).
+    No tokens: the call returns without launching anything."""
+    from omni_infer_amd import hip_ops as ops
+    E, n, H, I, lo, T = 64, 8, 512, 256, 56, 24
+    lay = Layer(n, H, I, seed=481, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    ra = _route_args(E, "noaux_tc")
+    g = gen(482)
+    x = tokens(T, H, 483).cuda()
+    logits = torch.randn(T, E, generator=g)
+    logits[:, lo:lo + n] = -30.0            # the local experts are never chosen
+    logits = logits.cuda()
+    a, b = _both(x, logits, None, ra, lo, n, d, shared, H, I)
+    _same(a, b, "nothing local, shared expert")
+    assert not bool(((a[2] >= lo) & (a[2] < lo + n)).any())
+    a, b = _both(x, logits, None, ra, lo, n, d, None, H, I)
+    _same(a, b, "nothing local, no shared expert")
+    assert not bool(b[0].float().abs().any())
+    out, w, ids = ops.moe_w8a8_layer_routed(x[:0], None, logits[:0], None, lo=lo, hi=lo + n, w13_packed=d["w13"],
+                                            w13_scale=d["s13"], w2_packed=d["w2"], w2_scale=d["s2"], shared=shared,
+                                            H=H, I=I, **ra)
+    assert tuple(out.shape) == (0, H) and tuple(ids.shape) == (0, 8)
