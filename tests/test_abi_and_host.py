@@ -74,6 +74,15 @@ def test_argument_validation_returns_codes(lib):
     assert lib.omni_moe_w8a8_layer(p, 0, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, 2, p,
                                    p, 1 << 30, None) == -1                                              # rows_dtype f16
     assert lib.omni_moe_w8a8_layer_workspace_bytes(4, 8, 32, 7168, 2048, 1, 2) == 0
+    # router and layer in one call: the router's checks come first, then the layer's
+    routed = lambda logits, E, n_group, T, rows_dtype: lib.omni_moe_w8a8_layer_routed(
+        p, 0, None, logits, None, E, n_group, 4, 1, 1, 0, 0, 1, 2.5, 1e-20, p, p, T, 8, 0, 32, p, p, p, p, None, None,
+        None, None, 7168, 2048, rows_dtype, p, p, 1 << 30, None)
+    assert routed(None, 256, 8, 4, 1) == -1 and b"null" in lib.omni_moe_last_error()
+    assert routed(p, 1024, 8, 4, 1) == -2                                                                # E > 512
+    assert routed(p, 256, 7, 4, 1) == -2 and b"n_group" in lib.omni_moe_last_error()
+    assert routed(p, 256, 8, 4, 2) == -1                                                                 # rows_dtype f16
+    assert routed(p, 256, 8, 0, 1) == 0                                                                  # empty batch
     assert lib.omni_moe_remap_ids(p, -1, p, 32, p, None) == -1
     assert lib.omni_moe_remap_ids(p, 8, None, 32, p, None) == -1
     assert lib.omni_moe_remap_ids(None, 0, None, 32, None, None) == 0                                    # nothing to do
