@@ -200,7 +200,7 @@ __global__ __launch_bounds__(NW * WAVE) void permute_single(PermArgs a) { permut
 // NW / 4 token rows of a block of NW wavefronts, four wavefronts a row: the row body of quant_rows.h with the
 // block barrier shared by the rows (rows past the end take part in it and touch no memory).
 template <int MAXV>
-__device__ __forceinline__ void quant_four_rows(const void* __restrict__ xv, int64_t r0, int64_t rows, int cols,
+__device__ __forceinline__ void quant_block_rows(const void* __restrict__ xv, int64_t r0, int64_t rows, int cols,
                                                 int8_t* __restrict__ q, float* __restrict__ scale, float* red) {
   const int tid = threadIdx.x & 255, qd = threadIdx.x >> 8;
   const int64_t r = r0 + qd;
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(NW * WAVE) void quant_permute_small(const void* __r
   constexpr int RPB = NW / 4;
   __shared__ float red[NW];
   const int quant_blocks = (int)((rows + RPB - 1) / RPB);
-  if ((int)blockIdx.x < quant_blocks) quant_four_rows<MAXV>(x, (int64_t)blockIdx.x * RPB, rows, cols, q, scale, red);
+  if ((int)blockIdx.x < quant_blocks) quant_block_rows<MAXV>(x, (int64_t)blockIdx.x * RPB, rows, cols, q, scale, red);
   else permute_single_body<NW>(a);
 }
 
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(NW * WAVE) void route_quant_permute_small(const voi
   __shared__ int s_last;
   const int route_blocks = (r.T + NW - 1) / NW;
   if ((int)blockIdx.x >= route_blocks) {
-    quant_four_rows<MAXV>(x, ((int64_t)blockIdx.x - route_blocks) * RPB, rows, cols, q, scale, red);
+    quant_block_rows<MAXV>(x, ((int64_t)blockIdx.x - route_blocks) * RPB, rows, cols, q, scale, red);
     return;
   }
   const int lane = threadIdx.x & (WAVE - 1);
