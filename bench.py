@@ -218,9 +218,26 @@ def bench_norm(args):
     print(json.dumps(result))
 
 
-def time_steps(fn, steps, warmup):
+PREHEAT_S = 0.3   # untimed, reported: the same step repeated for this long before the warm-up steps
+
+
+def preheat(fn, seconds=PREHEAT_S, max_steps=20000):
+    """Runs fn(i) untimed for about `seconds` of GPU time and returns the number of calls made.  A run of a few
+    dozen steps is over before the chip has left its idle clocks; with this in front, a short timed region
+    reads what a long one reads (the steady state of a serving loop)."""
+    n, t0 = 0, time.perf_counter()
+    while n < max_steps and time.perf_counter() - t0 < seconds:
+        for _ in range(16):
+            fn(n)
+            n += 1
+        torch.cuda.synchronize()
+    return n
+
+
+def time_steps(fn, steps, warmup, preheat_s=0.0):
     """Average GPU time of `steps` calls of fn(i) after `warmup` untimed ones (events on torch's current
     stream, which is the stream every library call is enqueued on), plus the host wall time per step."""
+    time_steps.last_preheat = preheat(fn, preheat_s) if preheat_s > 0 else 0
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
@@ -243,6 +260,32 @@ def single_step_spread(fn, n):
     torch.cuda.synchronize()
     per = sorted(a0.elapsed_time(a1) * 1e3 for a0, a1 in evs)
     return {"p10": per[int(0.1 * (n - 1))], "p50": per[(n - 1) // 2], "p90": per[int(0.9 * (n - 1))]}
+
+
+def graph_replay_us(step, n_sets, steps):
+    """The same steps replayed from a HIP graph (how a serving stack runs the decode path): one graph holds one
+    step per weight set, so the rotation of the eager loop is kept; average time of a step over the replays.
+    The capture runs on a stream of its own; the library calls record kernel launches only (no memset nodes)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for i in range(n_sets):
+            step(i)                       # per-device look-ups of the library happen outside the capture
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(n_sets):
+                step(i)
+    torch.cuda.current_stream().wait_stream(side)
+    replays = max(1, steps // n_sets)
+    preheat(lambda i: graph.replay(), PREHEAT_S / 3)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (replays * n_sets)
 
 
 def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_steps=None):
@@ -269,8 +312,10 @@ def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_ste
                                          out=out, rows_dtype=rows_dtype, topk_w=topk_w, topk_ids=topk_ids,
                                          **noaux_tc_routing(cfg))[0]
 
-    ms, wall_ms = time_steps(step, steps, warmup)
+    ms, wall_ms = time_steps(step, steps, warmup, PREHEAT_S)
+    preheat_steps = time_steps.last_preheat
     spread = single_step_spread(step, min(50, steps))
+    graph_us = graph_replay_us(step, len(sets), steps) if name == "decode" else None
 
     # routing actually produced (rows per local expert) for the byte / op counts
     w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
@@ -307,8 +352,8 @@ def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_ste
                                    H, I, M_cap, extra=(sets[0].sh13, sets[0].sh_s13), extra_rows=T, workspace=g1_ws,
                                    out=(hq, hs))                       # real int8 rows for GEMM2 to read
     ksteps = kernel_steps or max(10, steps // 2)
-    k1_ms, _ = time_steps(gemm1_only, ksteps, 5)
-    k2_ms, _ = time_steps(gemm2_only, ksteps, 5)
+    k1_ms, _ = time_steps(gemm1_only, ksteps, 5, PREHEAT_S / 3)
+    k2_ms, _ = time_steps(gemm2_only, ksteps, 5, PREHEAT_S / 3)
     name1 = ops.gemm_kernel_name(1, T, K, n_local, T, M_cap, H, I)
     name2 = ops.gemm_kernel_name(2, T, K, n_local, T, M_cap, H, I)
     rows_bytes = 4 if rows_dtype == torch.float32 else 2
@@ -337,7 +382,8 @@ def measure_layer(name, sets, steps, warmup, rows_dtype, no_cpu, dev, kernel_ste
         "workload": f"DeepSeek-V3-shape W8A8 MoE layer, {name}: {T} tokens, {n_local} local experts of {cfg['E']} + 1 shared, "
                     f"H={H}, I={I}, top-{K} grouped sigmoid routing",
         "tokens": T, "rows_routed": rows_routed, "active_groups": active, "rows_dtype": str(rows_dtype).split(".")[-1],
-        "layer_us": ms * 1e3, "ms_per_step": ms, "steps": steps, "warmup": warmup,
+        "layer_us": ms * 1e3, "ms_per_step": ms, "steps": steps, "warmup": warmup, "preheat_steps": preheat_steps,
+        "graph_us": graph_us,
         "algorithmic_bytes": layer_bytes, "algorithmic_ops": layer_ops,
         "hbm_frac": layer_bytes / (ms * 1e-3) / HBM_PEAK, "int8_frac": layer_ops / (ms * 1e-3) / INT8_PEAK,
         "host_wall_ms_per_step": wall_ms, "single_step_us": spread,
@@ -382,7 +428,7 @@ def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
                                          out=out, rows_dtype=rows_dtype, topk_w=topk_w, topk_ids=topk_ids,
                                          **noaux_tc_routing(cfg))[0]
 
-    ms, _ = time_steps(step, steps, warmup)
+    ms, _ = time_steps(step, steps, warmup, PREHEAT_S / 3)
 
     def step_routed_only(i):
         # the reference runs the shared expert on the rank's own tokens before the all-gather (deepseek_moe.py:244):
@@ -393,7 +439,7 @@ def measure_global_filter(sets, steps, warmup, rows_dtype, dev):
                                          out=out, rows_dtype=rows_dtype, topk_w=topk_w, topk_ids=topk_ids,
                                          **noaux_tc_routing(cfg))[0]
 
-    ms_routed, _ = time_steps(step_routed_only, steps, warmup)
+    ms_routed, _ = time_steps(step_routed_only, steps, warmup, PREHEAT_S / 3)
     w, ids, _ = ops.npu_moe_gating_top_k(logits, K, bias, cfg["topk_group"], cfg["n_group"], 1, 0, 1, cfg["scale"], 1e-20)
     counts = ops.moe_permute(ids, 0, n_local, L.OMNI_IDX_TOKEN_MAJOR).counts.cpu()
     rows_routed, active = int(counts.sum()), int((counts > 0).sum()) + 1
@@ -449,7 +495,7 @@ def measure_block(name, ws, steps, warmup, dev):
 
     def step(i):
         return blk(x, None, None, 3)
-    ms, wall_ms = time_steps(step, steps, warmup)
+    ms, wall_ms = time_steps(step, steps, warmup, PREHEAT_S / 3)
     ids = blk._route(x)[1]
     local = int(((ids >= 0) & (ids < n_local)).sum())
     return {"block_us": ms * 1e3, "host_wall_ms_per_step": wall_ms, "steps": steps, "local_assignments": local,
@@ -633,7 +679,8 @@ def main():
     head = dec if dec is not None else pre
     result = {
         "metric": "moe_layer_latency", "value": head["layer_us"], "unit": "us", "n_gpus": 1, "steps": head["steps"],
-        "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": False, "scaling": "weak",
+        "warmup": head["warmup"], "preheat_steps": head["preheat_steps"], "ms_per_step": head["ms_per_step"],
+        "graph_us": head["graph_us"], "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": head["workload"], "tokens": head["tokens"], "rows_routed": head["rows_routed"],
                    "active_groups": head["active_groups"], "weight_sets": len(sets), "rows_dtype": head["rows_dtype"]},
@@ -646,6 +693,7 @@ def main():
         result["cpu_baseline"] = head["cpu_baseline"]
     if dec is not None and pre is not None:
         result["prefill"] = {k: pre[k] for k in ("workload", "tokens", "rows_routed", "rows_dtype", "layer_us", "steps",
+                                                 "preheat_steps",
                                                  "algorithmic_ops", "int8_frac", "single_step_us", "roofline_gemm1",
                                                  "roofline_gemm2", "other_rows_dtype", "global_filter")}
         if "cpu_baseline" in pre:

@@ -15,7 +15,13 @@
  *    the host: all work is enqueued on `stream`, data dependent sizes (rows per
  *    expert) stay in device memory, so a call sequence can be captured in a HIP
  *    graph;
- *  - the library keeps no device state between calls.
+ *  - the library keeps no results between calls.  It does hold two static device
+ *    arrays on every GPU it runs on, from the first call that needs them until the
+ *    process ends: 16 KiB of arrival counters, zero between launches (see
+ *    omni_moe_w8a8_layer_routed), and the 64 MiB scratch of
+ *    omni_moe_w8a8_layer_static (resident whether that entry is used or not);
+ *  - measurement helpers (kernel names, hardware-rate probes, the tuning re-read)
+ *    are declared in omni_moe_diag.h, not here.
  *
  * Packed weight layout ("frag16"), produced by omni_moe_pack_weight
  *  A logical matrix B[Kdim][N] (Kdim = reduction dim, N = output channels) is
@@ -211,16 +217,6 @@ int omni_moe_gemm2_dequant(const int8_t* h_q, const float* h_scale, const int8_t
 size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int H, int I);
 
 /*
- * Which GEMM kernel the two entry points above launch for a call of these sizes (kind 1: GEMM1 with the
- * arguments of omni_moe_gemm1_swiglu_quant; kind 2: GEMM2, T and K unused), written to buf as the kernel's
- * template name, e.g. "gemm_stream<1,2,1,4>" or "gemm_pipe<2,4,lines>" (256 x 64*4 tile, line layout of the
- * activation operand; "frags": fragment layout).  A diagnostic for benchmarks and profiles
- * (no counterpart in the reference, whose kernels are chosen inside the closed operators).
- */
-int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, char* buf,
-                              size_t buf_bytes);
-
-/*
  * Expert placement (redundant copies of experts over the devices of an EP group).
  *
  * omni_placement_tables is HOST code on HOST pointers: from a placement pattern [world][layers][experts] of 0/1
@@ -248,39 +244,6 @@ int omni_placement_tables(const int32_t* pattern, int world, int layers, int exp
 int omni_moe_remap_ids(const int32_t* ids, int64_t n, const int32_t* map, int n_map, int32_t* out, void* stream);
 int omni_moe_record_activation(int64_t* counts, const int32_t* tokens_per_expert, int n, int64_t modulus,
                                void* stream);
-
-/*
- * The OMNI_MOE_* tuning variables (kernel choice, tile shape, split tiles ...) are read from the environment
- * once, at the first GEMM call of the process.  This reads them again: for tests and tuning runs that change
- * them inside one process.  Not to be called while another thread launches GEMMs.  No counterpart in the
- * reference.
- */
-void omni_moe_reload_tuning(void);
-
-/*
- * Diagnostic (no counterpart in the reference): the sustained rate of v_mfma_i32_32x32x32_i8 on given operand
- * bits with nothing else in the loop.  `blocks` blocks of 8 wavefronts each issue 8 * iters instructions per
- * wavefront (65 536 op each) on operands taken from `operands` (>= 64 KiB; zeros and random bits give different
- * rates because the chip lowers its clock with the switching activity).  The caller times the launch.
- */
-int omni_diag_mfma_i8_rate(const int8_t* operands, size_t operand_bytes, int iters, int blocks, int32_t* sink,
-                           void* stream);
-/*
- * Diagnostic (no counterpart in the reference): the int8 matrix instruction on the operand pattern of the tile
- * kernel (a 128 x 64 piece per wavefront, 128 accumulator registers, another operand pair from one instruction
- * to the next), as v_mfma_i32_32x32x32_i8 (form 32) or v_mfma_i32_16x16x64_i8 (form 16).  One pass of the loop is
- * 2 x 128 x 64 x 64 op per wavefront either way; `blocks` blocks of 8 wavefronts make `iters` passes.  The caller
- * times the launch: the two forms sustain different rates on the same operands.
- */
-int omni_diag_mfma_i8_tile_rate(const int8_t* operands, size_t operand_bytes, int form, int iters, int blocks,
-                                int32_t* sink, void* stream);
-/*
- * Diagnostic (no counterpart in the reference): `blocks` blocks of 256 threads read `bytes` of `buf` once, 16
- * bytes per lane and request, eight requests of a lane in flight, and do nothing else.  The caller times the
- * launch: bytes / time is what the memory system delivers to a kernel that only streams, the practical ceiling
- * of the weight-streaming GEMMs.
- */
-int omni_diag_hbm_read_rate(const void* buf, size_t bytes, int blocks, int32_t* sink, void* stream);
 
 /*
  * Weighted un-permute.  Replaces the routing half of npu_grouped_matmul_finalize_routing
@@ -324,11 +287,15 @@ size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int
  * topk_ids [T,K] int32 are outputs here and hold the routing when the call's work is done, everything else is
  * as for omni_moe_w8a8_layer, workspace size included.  Small calls (bf16 tokens, T*K <= 4096, H <= 8192) route,
  * quantise and sort in a single launch; other calls run the router's own launch first.
- *   The single launch counts its finished routing blocks in one of 256 arrival counters that the library keeps in
- *   static device memory (1 KiB per GPU, zero when the library is loaded).  Calls take the counters in turn and
- *   every launch leaves its counter at zero, so nothing is asked of the caller as long as fewer than 256 such
- *   calls are in flight on one GPU at a time.  The first such call on a device looks up that device's copy of the
- *   counters: make it outside a stream capture.
+ *   The single launch counts its finished routing blocks in an arrival counter, a word of a static device array
+ *   (16 KiB per GPU, zero when the library is loaded; every launch leaves its word at zero).  Eager calls take the
+ *   first 256 words in turn: nothing is asked of the caller as long as fewer than 256 such calls are in flight on
+ *   one GPU at a time.  A call recorded into a stream capture keeps its word for every replay, so it gets one that
+ *   eager calls never use: one word per (capture, stream) pair, shared by the calls that stream records into that
+ *   capture (they are ordered in every replay; a graph does not run concurrently with itself).  3840 such words
+ *   exist; when they are used up, or when the first such call on a device happens inside a capture (the look-up
+ *   of the device's copy of the array is not made there), the call records the separate launches instead: same
+ *   results, one launch more.
  */
 int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const float* x_scale_in, const float* logits,
                                const float* bias, int E, int n_group, int topk_group, int score_fn, int group_mode,
@@ -338,6 +305,31 @@ int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const float* x_scale_
                                const float* w2_scale, const int8_t* sh13_packed, const float* sh13_scale,
                                const int8_t* sh2_packed, const float* sh2_scale, int H, int I, int rows_dtype,
                                void* out_bf16, void* workspace, size_t ws_bytes, void* stream);
+
+/*
+ * The whole MoE block in one call: gate projection, router and layer, i.e. self.gate.forward(hidden_states.float())
+ * + FusedMoE.select_experts + the quant method's apply + the sum with the shared expert
+ * (omni/models/common/layers/moe/deepseek_moe.py:147-152, 244-263, 303, 323-339, 366).  The results are those of
+ * omni_moe_gate_route followed by omni_moe_w8a8_layer, bit for bit.
+ *   x [T,H] is what the gate reads (x_dtype BF16 or F32); gate_w [E,H] fp32 or bf16 (gate_w_dtype); the routing
+ *   arguments, round_logits_bf16, topk_w / topk_ids (outputs) as for omni_moe_gate_route.
+ *   x_q / x_scale (both or neither): the tokens already quantised (the producer in front of the block can make
+ *   them, omni_add_rms_norm_quant); without them x must be bf16 and is quantised here.
+ *   Everything from T on as for omni_moe_w8a8_layer.  workspace: omni_moe_w8a8_block_workspace_bytes.
+ * Two launches stand in front of the GEMMs for small calls (at most 1024 assignments): the partial sums of the
+ * gate projection, then one launch that adds them up, routes, quantises and sorts (its arrival counter: see
+ * omni_moe_w8a8_layer_routed); larger calls run the router, the quantiser and the sort as launches of their own.
+ */
+int omni_moe_w8a8_block(const void* x, int x_dtype, const int8_t* x_q, const float* x_scale, const void* gate_w,
+                        int gate_w_dtype, const float* bias, int E, int n_group, int topk_group, int score_fn,
+                        int group_mode, int masked_fill_zero, int weight_from_c, int renorm, float scale, float eps,
+                        int round_logits_bf16, float* topk_w, int32_t* topk_ids, int T, int K, int lo, int hi,
+                        const int8_t* w13_packed, const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
+                        const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
+                        const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16, void* workspace,
+                        size_t ws_bytes, void* stream);
+size_t omni_moe_w8a8_block_workspace_bytes(int T, int K, int n_local, int H, int I, int E, int with_shared,
+                                           int rows_dtype);
 
 /*
  * The same layer on the library's own scratch.  No counterpart in the reference: it is for callers

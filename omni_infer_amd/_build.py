@@ -5,6 +5,8 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -16,10 +18,11 @@ SOURCES = ["route.hip", "quant.hip", "norm.hip", "permute.hip", "gemm.hip", "com
 # The packed-fp32 feature is switched off for the device pass; the host pass does not know it
 # and says so, which is harmless.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
+NOISE = "is not a recognized feature for this target"
 
 
 def hipcc_path() -> str:
@@ -29,18 +32,27 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (set HIPCC)")
 
 
-def build(verbose: bool = True) -> str:
-    """Always compiles; returns the path of the shared library."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", LIB_PATH + ".tmp", *[os.path.join(CSRC, s) for s in SOURCES]]
+def _run(cmd, verbose):
     if verbose:
         print("[omni_infer_amd] " + " ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    err = "\n".join(l for l in res.stderr.splitlines() if NOISE not in l)
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
+        raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose: bool = True) -> str:
+    """Always compiles (every source to an object of its own, side by side, then one link); returns
+    the path of the shared library."""
+    hipcc = hipcc_path()
+    with tempfile.TemporaryDirectory(prefix="omni_moe_build_") as tmp:
+        objs = [os.path.join(tmp, s.replace(".hip", ".o")) for s in SOURCES]
+        jobs = [[hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
+        with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+            list(pool.map(lambda c: _run(c, verbose), jobs))
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH + ".tmp", *objs], verbose)
     os.replace(LIB_PATH + ".tmp", LIB_PATH)
     return LIB_PATH
 

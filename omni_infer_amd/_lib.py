@@ -44,6 +44,9 @@ SIGNATURES = {
     "omni_moe_w8a8_layer_workspace_bytes": (c_size_t, [I, I, I, I, I, I, I]),
     "omni_moe_w8a8_layer_routed": (I, [P, I, P, P, P, I, I, I, I, I, I, I, I, c_float, c_float, P, P, I, I, I, I,
                                        P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
+    "omni_moe_w8a8_block": (I, [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, c_float, c_float, I, P, P, I, I, I, I,
+                                P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
+    "omni_moe_w8a8_block_workspace_bytes": (c_size_t, [I, I, I, I, I, I, I, I]),
     "omni_moe_w8a8_layer_static": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, I, P, P]),
 }
 
@@ -55,7 +58,7 @@ OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 
 OMNI_STATIC_SCRATCH_BYTES = 64 << 20
-ABI_VERSION = 6   # omni_moe_abi_version() of the header these signatures were written from
+ABI_VERSION = 7   # omni_moe_abi_version() of the header these signatures were written from
 
 _lib = None
 

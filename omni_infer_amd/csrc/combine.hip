@@ -18,7 +18,7 @@ void omni_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 extern "C" const char* omni_moe_last_error(void) { return g_err; }
-extern "C" int omni_moe_abi_version(void) { return 6; }
+extern "C" int omni_moe_abi_version(void) { return 7; }
 
 namespace {
 
@@ -218,41 +218,9 @@ extern "C" int omni_moe_combine(const void* rows, int rows_dtype, const float* t
 }
 
 // ---------------------------------------------------------------- whole layer
-namespace {
-struct LayerWs {
-  size_t x_q, x_s, sorted_src, src_to_dst, counts, offsets, perm_ws, h_q, h_s, g1_ws, rows, total;
-  size_t perm_bytes, g1_bytes;
-  int64_t M_cap;
-  int rows_dtype;
-};
-// rows_dtype: the caller's choice for the expert rows between GEMM2 and the combine, fp32 (the
-// numerics of the fused GEMM2+finalize operator) or bf16 (those of the separate GEMM2 and finalize
-// operators, half the bytes of the largest intermediate).
-LayerWs layer_layout(int T, int K, int G, int H, int I, int with_shared, int rows_dtype) {
-  LayerWs L{};
-  L.M_cap = (int64_t)T * K + (with_shared ? T : 0);
-  size_t o = 0;
-  auto take = [&](size_t bytes) { size_t at = o; o += align256(bytes); return at; };
-  L.x_q = take((size_t)T * H);
-  L.x_s = take((size_t)T * 4);
-  L.sorted_src = take((size_t)T * K * 4);
-  L.src_to_dst = take((size_t)T * K * 4);
-  L.counts = take((size_t)G * 4);
-  L.offsets = take((size_t)(G + 1) * 4);
-  L.perm_bytes = omni_moe_permute_workspace_bytes(T, K, G);
-  L.perm_ws = take(L.perm_bytes);
-  L.h_q = take((size_t)L.M_cap * I);
-  L.h_s = take((size_t)L.M_cap * 4);
-  L.g1_bytes = omni_moe_gemm1_workspace_bytes(T, K, G, with_shared ? T : 0, L.M_cap, H, I);
-  const size_t g2_bytes = omni_moe_gemm2_workspace_bytes(G, with_shared ? T : 0, L.M_cap, H, I);
-  if (g2_bytes > L.g1_bytes) L.g1_bytes = g2_bytes;
-  L.g1_ws = take(L.g1_bytes);
-  L.rows_dtype = rows_dtype;
-  L.rows = take((size_t)L.M_cap * H * (L.rows_dtype == OMNI_DT_F32 ? 4 : 2));
-  L.total = o;
-  return L;
-}
-}  // namespace
+// byte offsets of the parts of the caller's workspace: omni_host::layer_layout (host_logic.h)
+using omni_host::LayerWs;
+using omni_host::layer_layout;
 
 extern "C" size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared,
                                                       int rows_dtype) {
@@ -296,21 +264,21 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
   size_t tail_bytes = 0;
   void* const tail = omni_tile_tail_area(T, K, G, extra, L.M_cap, H, I, ws + L.g1_ws, L.g1_bytes, &cnt_words, &tail_bytes);
   bool routed = route == nullptr;
-  if (route != nullptr && x_dtype == OMNI_DT_BF16) {
-    // routing, quantisation and sort in one launch when the call is small
-    rc = omni_route_quant_permute_fused(route, x, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), K, lo, hi, sorted_src,
-                                        src_to_dst, (int32_t*)(ws + L.counts), offsets, (int32_t*)tail, cnt_words, stream);
+  if (route != nullptr && (x_dtype == OMNI_DT_BF16 || x_dtype == -1)) {
+    // routing, quantisation (of bf16 tokens) and sort in one launch when the call is small
+    const bool quantise = x_dtype == OMNI_DT_BF16;
+    rc = omni_route_quant_permute_fused(route, quantise ? x : nullptr, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), K,
+                                        lo, hi, sorted_src, src_to_dst, (int32_t*)(ws + L.counts), offsets, (int32_t*)tail,
+                                        cnt_words, stream);
     if (rc < 0) return rc;
     routed = sorted = rc == 0;
-    if (sorted) {
+    if (sorted && quantise) {
       xq = (const int8_t*)(ws + L.x_q);
       xs = (const float*)(ws + L.x_s);
     }
   }
   if (!routed) {
-    rc = omni_moe_route(route->logits, route->bias, T, route->E, route->n_group, route->topk_group, K, route->score_fn,
-                        route->group_mode, route->masked_fill_zero, route->weight_from_c, route->renorm, route->scale,
-                        route->eps, route->topk_w, route->topk_ids, stream);
+    rc = omni_route_launch(route, T, K, stream);
     if (rc) return rc;
   }
   if (x_dtype != -1 && !sorted) {
@@ -388,6 +356,49 @@ extern "C" int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const floa
   return layer_impl(x, x_dtype, x_scale_in, topk_w, topk_ids, &rp, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
                     w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, workspace,
                     ws_bytes, stream);
+}
+
+// ---------------------------------------------------------------- the whole block: gate, router, layer
+extern "C" size_t omni_moe_w8a8_block_workspace_bytes(int T, int K, int n_local, int H, int I, int E, int with_shared,
+                                                      int rows_dtype) {
+  const size_t layer = omni_moe_w8a8_layer_workspace_bytes(T, K, n_local, H, I, with_shared, rows_dtype);
+  const size_t gate = omni_moe_gate_route_workspace_bytes(T, H, E);
+  if (layer == 0 || (gate == 0 && T > 0)) return 0;
+  return align256(layer) + gate;
+}
+
+extern "C" int omni_moe_w8a8_block(const void* x, int x_dtype, const int8_t* x_q, const float* x_scale, const void* gate_w,
+                                   int gate_w_dtype, const float* bias, int E, int n_group, int topk_group, int score_fn,
+                                   int group_mode, int masked_fill_zero, int weight_from_c, int renorm, float scale,
+                                   float eps, int round_logits_bf16, float* topk_w, int32_t* topk_ids, int T, int K, int lo,
+                                   int hi, const int8_t* w13_packed, const float* w13_scale, const int8_t* w2_packed,
+                                   const float* w2_scale, const int8_t* sh13_packed, const float* sh13_scale,
+                                   const int8_t* sh2_packed, const float* sh2_scale, int H, int I, int rows_dtype,
+                                   void* out_bf16, void* workspace, size_t ws_bytes, void* stream) {
+  if (T < 0 || E <= 0 || K <= 0 || H <= 0 || I <= 0 || hi <= lo) OMNI_FAIL(OMNI_E_INVALID, "block: bad sizes T=%d E=%d K=%d", T, E, K);
+  if (T == 0) return OMNI_OK;
+  if (!x || !gate_w || !topk_w || !topk_ids || !workspace) OMNI_FAIL(OMNI_E_INVALID, "block: null pointer");
+  if ((x_q == nullptr) != (x_scale == nullptr)) OMNI_FAIL(OMNI_E_INVALID, "block: quantised tokens and their scales come together");
+  if (x_q == nullptr && x_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_UNSUPPORTED, "block: tokens that are not quantised yet must be bf16");
+  if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "block: rows_dtype %d", rows_dtype);
+  if ((uintptr_t)workspace % 256) OMNI_FAIL(OMNI_E_INVALID, "block: workspace must be 256-byte aligned");
+  int rc = omni_route_check("block", T, E, n_group, topk_group, K, score_fn);
+  if (rc) return rc;
+  const int with_shared = sh13_packed != nullptr;
+  const size_t layer_bytes = align256(omni_moe_w8a8_layer_workspace_bytes(T, K, hi - lo, H, I, with_shared, rows_dtype));
+  const size_t gate_bytes = omni_moe_gate_route_workspace_bytes(T, H, E);
+  if (gate_bytes == 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "block: the gate projection needs H %% 128 == 0 (H=%d)", H);
+  if (ws_bytes < layer_bytes + gate_bytes) OMNI_FAIL(OMNI_E_WORKSPACE, "block: workspace %zu < %zu", ws_bytes, layer_bytes + gate_bytes);
+  char* gate_ws = (char*)workspace + layer_bytes;
+  OmniRouteParams rp{nullptr, bias, E, n_group, topk_group, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm,
+                     scale, eps, topk_w, topk_ids};
+  rc = omni_gate_partials(x, x_dtype, gate_w, gate_w_dtype, T, H, E, gate_ws, gate_bytes, &rp.n_parts, &rp.group_len, stream);
+  if (rc) return rc;
+  rp.partials = (const float*)gate_ws;
+  rp.round_logits_bf16 = round_logits_bf16;
+  return layer_impl(x_q ? (const void*)x_q : x, x_q ? -1 : x_dtype, x_scale, topk_w, topk_ids, &rp, T, K, lo, hi, w13_packed,
+                    w13_scale, w2_packed, w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16,
+                    workspace, layer_bytes, stream);
 }
 
 // ---------------------------------------------------------------- whole layer on the library's own scratch

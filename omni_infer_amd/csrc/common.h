@@ -6,6 +6,7 @@
 #include <stdarg.h>
 
 #include "../../include/omni_moe_hip.h"
+#include "../../include/omni_moe_diag.h"
 
 // Every floating-point operation below is meant to round once: no contraction into FMA.
 #pragma clang fp contract(off)
@@ -16,15 +17,10 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 #define WAVE 64
 
-inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
-
-// ---------------------------------------------------------------- host side error state
-void omni_set_error(const char* fmt, ...);
-#define OMNI_FAIL(code, ...)        \
-  do {                              \
-    omni_set_error(__VA_ARGS__);    \
-    return (code);                  \
-  } while (0)
+// ---------------------------------------------------------------- host side error state, host-side integer logic
+// (omni_set_error, OMNI_FAIL, align256, kernel choice, tile numbering, workspace layout: host_logic.h)
+#include "host_logic.h"
+using omni_host::align256;
 #define OMNI_CHECK_LAUNCH(what)                                                            \
   do {                                                                                     \
     hipError_t e__ = hipGetLastError();                                                    \
@@ -45,9 +41,22 @@ struct OmniRouteParams {
   float scale, eps;
   float* topk_w;
   int32_t* topk_ids;
+  // instead of the logits: the partial sums of the gate projection [n_parts][T][E] (omni_gate_partials), added
+  // up in groups of group_len, and what is done with the finished logits
+  const float* partials = nullptr;
+  int n_parts = 0, group_len = 1, round_logits_bf16 = 0;
+  float* logits_out = nullptr;
 };
 // library-internal: the argument checks of omni_moe_route (route.hip)
 int omni_route_check(const char* what, int T, int E, int n_group, int topk_group, int K, int score_fn);
+// library-internal (route.hip): the router as a launch of its own, on the logits or on the partial sums of rp
+int omni_route_launch(const OmniRouteParams* rp, int T, int K, void* stream);
+// library-internal (route.hip): the partial sums of the gate projection of omni_moe_gate_route into `partials`
+// (omni_moe_gate_route_workspace_bytes(T, H, E) bytes); how many parts there are and how they are grouped
+int omni_gate_partials(const void* x, int x_dtype, const void* gate_w, int w_dtype, int T, int H, int E, void* partials,
+                       size_t partials_bytes, int* n_parts, int* group_len, void* stream);
+// library-internal: most groups of partial sums the launch that also routes, quantises and sorts takes
+constexpr int OMNI_FOLD_MAX_GROUPS = 16;
 // library-internal: routing, bf16 row quantisation and assignment sort in one launch (permute.hip); 1 = not
 // applicable.  zero_words as above.
 int omni_route_quant_permute_fused(const OmniRouteParams* rp, const void* x_bf16, int T, int H, int8_t* q, float* scale,
@@ -335,16 +344,9 @@ struct RowBlockKinds {
   int total_h, total_l;
   bool small;
 };
-// A group's last block is light when it has at most light_max rows -- except in a group of exactly one full block
-// and a few rows more: there the small block stays next to the full one, whose weight panel it shares (deferred
-// to the end it would fetch that panel a second time, and with one full block per group that doubles the traffic).
-__device__ __forceinline__ bool last_block_is_light(int c, int BM, int light_max) {
-  return (c % BM) > 0 && (c % BM) <= light_max && c / BM != 1;
-}
-__device__ __forceinline__ int heavy_blocks(int c, int BM, int light_max) {
-  return c / BM + ((c % BM) > 0 && !last_block_is_light(c, BM, light_max));
-}
-__device__ __forceinline__ int light_blocks(int c, int BM, int light_max) { return last_block_is_light(c, BM, light_max); }
+using omni_host::heavy_blocks;
+using omni_host::last_block_is_light;
+using omni_host::light_blocks;
 __device__ __forceinline__ RowBlockKinds row_block_kinds_scan(const int32_t* __restrict__ offsets, int G, int extra_rows,
                                                               int BM, int light_max) {
   const int lane = threadIdx.x & (WAVE - 1);

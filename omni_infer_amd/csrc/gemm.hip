@@ -699,72 +699,11 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
   }
 }
 
-// ---- which tile a block id names (shared by the tile kernels)
-// Real tiles (row blocks that exist x column tiles) get the ids [0, n_real): first the tiles of the heavy row
-// blocks, then those of the light ones; the last `left` real tiles (a last partial round of at most half the
-// chip) are each split `split` ways along the reduction, the helper shares have the ids [n_real, total).
-struct TileCount { int n_heavy, n_real, left, split, total; };
-struct TileSel { int bx, by, share, tail_tile; bool light; };
-[[maybe_unused]] constexpr int TILE_LIGHT_MAX = 96;
-
-template <bool LINES>
-__device__ __forceinline__ TileCount tile_count(const GemmArgs& a, int total_h, int total_l, int nk_all) {
-  TileCount t;
-  t.n_heavy = total_h * a.tile_gx;
-  t.n_real = (total_h + total_l) * a.tile_gx;
-  t.left = 0;
-  t.split = 1;
-  if (a.tail_part != nullptr && a.tile_slots > 0) {
-    t.left = t.n_real % a.tile_slots;
-    if (t.left > 0 && 2 * t.left <= a.tile_slots)
-      t.split = min(min(a.tile_split_max, a.tile_slots / t.left), LINES ? nk_all / 2 : nk_all);
-    if (t.split < 2) { t.split = 1; t.left = 0; }
-  }
-  t.total = t.n_real + t.left * (t.split - 1);
-  return t;
-}
-
-// false: the id names no work
-__device__ __forceinline__ bool tile_select(const GemmArgs& a, const TileCount& tc, int total_h, int total_l, int id,
-                                            TileSel& s) {
-  constexpr int TILE_PR = 4;
-  const int gx = a.tile_gx, pc = a.tile_pc, npc = gx / pc, per_patch = TILE_PR * pc;
-  s.share = 0;
-  s.tail_tile = -1;
-  if (id >= tc.n_real) {
-    const int h = id - tc.n_real;
-    if (tc.split == 1 || h >= tc.left * (tc.split - 1)) return false;
-    s.tail_tile = h / (tc.split - 1);
-    s.share = 1 + h % (tc.split - 1);
-    id = tc.n_real - tc.left + s.tail_tile;
-  } else if (tc.split > 1 && id >= tc.n_real - tc.left) {
-    s.tail_tile = id - (tc.n_real - tc.left);
-  }
-  s.light = id >= tc.n_heavy;
-  const int t = s.light ? id - tc.n_heavy : id;   // id inside the set
-  const int RB = s.light ? total_l : total_h;     // row blocks of the set
-  const int bulk_rows = RB / TILE_PR * TILE_PR;
-  const int patches = bulk_rows / TILE_PR * npc, patches8 = patches / 8 * 8;
-  const int nA = patches8 * per_patch, nB = (patches - patches8) * per_patch;
-  if (t < nA + nB) {
-    int patch, q;
-    if (t < nA) {
-      // the tiles of a patch are 8 ids apart: one XCD runs them all
-      const int j = t >> 3;
-      patch = (j / per_patch) * 8 + (t & 7);
-      q = j % per_patch;
-    } else {
-      patch = patches8 + (t - nA) / per_patch;
-      q = (t - nA) % per_patch;
-    }
-    s.by = (patch / npc) * TILE_PR + q / pc;
-    s.bx = (patch % npc) * pc + q % pc;
-  } else {
-    s.by = bulk_rows + (t - nA - nB) / gx;
-    s.bx = (t - nA - nB) % gx;
-  }
-  return true;
-}
+// ---- which tile a block id names: omni_host::tile_count / tile_select (host_logic.h)
+using omni_host::TileCount;
+using omni_host::TileGeom;
+using omni_host::TileSel;
+using omni_host::TILE_LIGHT_MAX;
 
 // Hand-over between the shares of a split tile (their blocks may run on different XCDs, each with its own
 // L2).  Every wavefront stores its partial sums, all wavefronts meet at the block barrier, then one
@@ -857,9 +796,10 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   constexpr int LIGHT_MAX = TILE_LIGHT_MAX;
   const RowBlockKinds scan = row_block_kinds_scan(a.offsets, a.G, a.extra_rows, BM, LIGHT_MAX);
   const int nk_all = a.Kdim / 64;
-  const TileCount tc = tile_count<LINES>(a, scan.total_h, scan.total_l, nk_all);
+  const TileGeom geom{a.tile_gx, a.tile_pc, a.tile_slots, a.tile_split_max, a.tail_part != nullptr};
+  const TileCount tc = omni_host::tile_count(geom, scan.total_h, scan.total_l, LINES ? nk_all / 2 : nk_all);
   TileSel sel;
-  if (!tile_select(a, tc, scan.total_h, scan.total_l, (int)blockIdx.x, sel)) return;
+  if (!omni_host::tile_select(geom, tc, scan.total_h, scan.total_l, (int)blockIdx.x, sel)) return;
   const int bx = sel.bx, by = sel.by, split = tc.split, share = sel.share, tail_tile = sel.tail_tile;
   const bool light = sel.light;
   RowBlock rb;
@@ -867,8 +807,8 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   // this block's k-steps [k_first, k_first + nk64)
   // (shares of the line layout begin and end on whole super-steps of 128)
   constexpr int KU = LINES ? 2 : 1;
-  const int k_first = (tail_tile >= 0) ? share * (nk_all / KU) / split * KU : 0;
-  const int k_end = (tail_tile >= 0) ? (share + 1) * (nk_all / KU) / split * KU : nk_all;
+  int k_first = 0, k_end = nk_all;
+  if (tail_tile >= 0) omni_host::tile_share_k_range(nk_all, KU, split, share, k_first, k_end);
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int nk64 = k_end - k_first;
   const int I = (KIND == 1) ? a.N / 2 : 0;
@@ -1074,134 +1014,21 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(const int8_t* __restri
 }
 
 // ---------------------------------------------------------------- host side dispatch
-struct Plan {
-  bool tile;
-  int mt, nt, d;  // stream kernel parameters
-  int S;          // k splits (GEMM1 stream kernel only)
-  int64_t per;    // expected rows of a busy group
-};
-
-// Tuning aids, read from the environment once (the first GEMM call of the process) and never again:
-//   OMNI_MOE_FORCE_KERNEL  1 stream kernel, 2 tile kernel, whatever the row counts
-//   OMNI_MOE_G1 / _G2      "mt,nt,d[,S]" of the stream kernel of GEMM1 / GEMM2; a combination that is not
-//                          compiled in is refused here, with a message, and the default is used
-//   OMNI_MOE_TILE_WN       2: tile kernel of 256 x 128 instead of 256 x 256
-//   OMNI_MOE_TILE_LINES    0: the 256 x 256 tile kernel keeps the fragment layout of the activation operand
-//   OMNI_MOE_TILE_MFMA16   0: the line-layout tile kernel multiplies with v_mfma_i32_32x32x32_i8 instead of 16x16x64
-//   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
-//   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
-//   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
-//   OMNI_MOE_EQUAL_PROGRESS bit 0: the stream kernel of GEMM1 lowers the issue priority of its wavefronts as they
-//                          advance (default 1), bit 1: that of GEMM2 too (measured slower in every geometry)
-struct Tuning {
-  int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
-  int tile_mfma16 = 1;
-  bool have[3] = {false, false, false};
-  int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
-};
-bool stream_variant_exists(int kind, int mt, int nt, int d);
-Tuning read_tuning() {
-  Tuning r;
-  auto geti = [](const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : dflt;
-  };
-  r.force_kernel = geti("OMNI_MOE_FORCE_KERNEL", 0);
-  r.tile_wn = geti("OMNI_MOE_TILE_WN", 4);
-  r.tile_tail = geti("OMNI_MOE_TILE_TAIL", 1);
-  r.tile_mfma16 = geti("OMNI_MOE_TILE_MFMA16", 1);
-  r.tile_split = geti("OMNI_MOE_TILE_SPLIT", 4);
-  r.rowq = geti("OMNI_MOE_ROWQ", 0);
-  r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
-  r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
-  for (int kind = 1; kind <= 2; ++kind) {
-    const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
-    const char* e = getenv(name);
-    if (!e) continue;
-    int mt = 0, nt = 0, d = 0, S = 0;
-    if (sscanf(e, "%d,%d,%d,%d", &mt, &nt, &d, &S) >= 3 && stream_variant_exists(kind, mt, nt, d)) {
-      r.have[kind] = true;
-      r.mt[kind] = mt; r.nt[kind] = nt; r.d[kind] = d; r.S[kind] = S;
-    } else {
-      fprintf(stderr, "omni_moe: %s=\"%s\" names no compiled stream kernel; ignored\n", name, e);
-    }
-  }
-  return r;
-}
-// read at the first GEMM call of the process; omni_moe_reload_tuning() reads the environment again
-Tuning& tuning_store() {
-  static Tuning t = read_tuning();
-  return t;
-}
-const Tuning& tuning() { return tuning_store(); }
-
-// the compiled (KIND, MT, NT, D) combinations of gemm_stream
-#define OMNI_STREAM_VARIANTS(X)                                                        \
-  X(1, 1, 1, 4) X(1, 2, 1, 4) X(1, 4, 1, 4) X(1, 1, 1, 8) X(1, 2, 1, 8)                \
-  X(1, 1, 2, 4) X(1, 2, 2, 4) X(1, 4, 2, 4) X(1, 2, 2, 8)                              \
-  X(2, 1, 1, 4) X(2, 2, 1, 4) X(2, 4, 1, 4) X(2, 1, 2, 4) X(2, 2, 2, 4) X(2, 4, 2, 4)  \
-  X(2, 1, 4, 4) X(2, 2, 4, 4) X(2, 2, 2, 8) X(2, 1, 2, 8) X(2, 2, 1, 8)
-bool stream_variant_exists(int kind, int mt, int nt, int d) {
-#define HAS(K_, MT_, NT_, D_) if (kind == K_ && mt == MT_ && nt == NT_ && d == D_) return true;
-  OMNI_STREAM_VARIANTS(HAS)
-#undef HAS
-  return false;
-}
-
-// Decides the kernel from what the host knows: the expected rows of a busy group.  The stream
-// kernel covers a group with blocks of 16*mt rows; GEMM1 is also split along k so that the
-// launch has several times more blocks than the chip has block slots (no idle tail).
+// kernel choice (make_plan), tuning variables, workspace sizes: host_logic.h
+using omni_host::Plan;
+using omni_host::Tuning;
+using omni_host::tuning;
+using omni_host::tile_lines;
+using omni_host::tile_wn;
+using omni_host::TILE_TAIL_BYTES;
+using omni_host::TILE_TAIL_CNT_BYTES;
+using omni_host::TILE_TAIL_CNT_WORDS;
+using omni_host::TILE_TAIL_PART_BYTES;
+using omni_host::gemm1_ws_bytes;
 template <int KIND>
 Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_cap) {
-  const int units = (KIND == 1) ? N / 32 : N / 16;  // KIND 1: (gate, up) strip pairs; KIND 2: strips
-  // expected rows of a routed group (uniform routing); the shared group, when there is one, has T rows
-  int64_t avg = (G > 0) ? ((int64_t)T * K + G - 1) / G : 0;
-  if (avg > (int64_t)T) avg = T;
-  const int64_t per = (G > 0) ? avg : extra_rows;
-  Plan p{};
-  p.per = per;
-  // Measured on the DeepSeek-V3 shape (32 routed groups + the shared one): up to 56 expected rows per
-  // routed group the stream kernel wins (row blocks of 64 rows from 25 expected rows on, so that
-  // nearly every group is one block and its weights are read once; the shared group then takes a few
-  // blocks and re-reads its 3 % of the bytes); above that the tile kernel does.
-  p.tile = (G > 0) ? per > 56 : per > 128;
-  const Tuning& tn = tuning();
-  const int force = tn.force_kernel;
-  if (force == 1) p.tile = false;
-  if (force == 2) p.tile = true;
-  const bool tile_ok = units % ((KIND == 1) ? 4 : 8) == 0;  // the tile kernel takes 64 / 128 channels at least
-  if (p.tile && !tile_ok) p.tile = false;
-  // the stream kernel walks the reduction in chunks of 256: other lengths go to the tile kernel
-  if (!p.tile && Kdim % 256 != 0 && tile_ok && force != 1) p.tile = true;
-  p.mt = per <= 10 ? 1 : (per <= 24 ? 2 : 4);
-  p.S = 1;
-  if (KIND == 1) {
-    p.nt = 1; p.d = 4;
-  } else {
-    p.nt = 1; p.d = 4;
-  }
-  int s_env = 0;
-  if (tn.have[KIND]) { p.mt = tn.mt[KIND]; p.nt = tn.nt[KIND]; p.d = tn.d[KIND]; s_env = tn.S[KIND]; }
-  if (Kdim % (64 * p.d) != 0) p.d = 4;
-  if (KIND == 1 && !p.tile && Kdim % 256 == 0 && units % (4 * p.nt) == 0) {
-    const int nchunks = Kdim / 256, dc = p.d / 4;
-    const int Gt = G + (extra_rows > 0 ? 1 : 0);
-    int64_t mb = (int64_t)Gt * ((per + 16 * p.mt - 1) / (16 * p.mt));
-    int64_t base = (int64_t)(units / (4 * p.nt)) * (mb > 0 ? mb : 1);
-    // measured on MI355X: extra k splits cost more in block start-up than they win back in the
-    // tail of the launch, so the default is one share (the tuning aid OMNI_MOE_G1 can ask for more)
-    int want = 1;
-    (void)base;
-    if (s_env > 0) want = s_env;
-    int best = 1;
-    for (int sdiv = 1; sdiv <= nchunks; ++sdiv) {
-      if (nchunks % sdiv != 0 || (nchunks / sdiv) % dc != 0 || nchunks / sdiv < 2 * dc) continue;
-      if (sdiv <= want) best = sdiv;
-    }
-    p.S = best;
-  }
   (void)M_cap;
-  return p;
+  return omni_host::make_plan(KIND, T, K, G, extra_rows, Kdim, N);
 }
 
 template <int KIND, int MT, int NT, int D>
@@ -1216,24 +1043,6 @@ void launch_stream(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st)
   dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks, (unsigned)a.S), block(256);
   hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
 }
-
-// the line layout of the activation operand needs whole super-steps of 128 (OMNI_MOE_TILE_LINES=0: never)
-bool tile_lines(int Kdim) { return tuning().tile_lines && Kdim % 128 == 0; }
-
-// wavefront columns of the large tile: 4 (256 channels per block) when the channel count allows, else 2
-int tile_wn(int kind, int units) {
-  const int wide = (kind == 1) ? 8 : 16;  // units per 256-channel block
-  return (tuning().tile_wn == 4 && units % wide == 0) ? 4 : 2;
-}
-
-// Scratch of the split tiles of a launch: arrival counters, then one slot of partial accumulators per
-// share.  At most `tile_slots` shares exist (splits x split tiles <= slots), a slot is the 256 x 64*WN
-// int32 tile of a block, and the slot count is capped so that the area has one size for every shape.
-// (the counters of GEMM1 and of GEMM2 are different words, so that one clearing in front of both launches serves)
-constexpr int TILE_TAIL_CNT_WORDS = 1024;                                  // per kind of GEMM
-constexpr size_t TILE_TAIL_CNT_BYTES = 2 * TILE_TAIL_CNT_WORDS * sizeof(int32_t);
-constexpr size_t TILE_TAIL_PART_BYTES = (size_t)64 << 20;
-constexpr size_t TILE_TAIL_BYTES = TILE_TAIL_CNT_BYTES + TILE_TAIL_PART_BYTES;
 
 __global__ void zero_words_kernel(int32_t* p, int n) {
   for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0;
@@ -1325,14 +1134,6 @@ int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, void* tail_ws
   return OMNI_OK;
 }
 
-size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
-  if (p.tile) {
-    // y = silu(gate) * up before the row quantiser, then the scratch of the split tiles
-    return align256((size_t)M_cap * I * sizeof(float) + 256) + TILE_TAIL_BYTES;
-  }
-  return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
-}
-
 void launch_quant_rows_y(const float* y, const int32_t* offsets, int G, int extra_rows, int I, int64_t M_cap,
                          int8_t* h_q, float* h_scale, hipStream_t st) {
   dim3 qgrid((unsigned)((M_cap + 3) / 4)), qblock(256);
@@ -1355,9 +1156,7 @@ int check_group_args(const char* what, const int32_t* offsets, int G, int H, int
 }  // namespace
 
 extern "C" size_t omni_moe_gemm1_workspace_bytes(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I) {
-  if (M_cap < 0 || I <= 0 || H <= 0 || T < 0 || K <= 0 || G < 0) return 0;
-  Plan p = make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap);
-  return gemm1_ws_bytes(p, M_cap, I);
+  return omni_host::gemm1_workspace_bytes(T, K, G, extra_rows, M_cap, H, I);
 }
 
 extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src,
@@ -1479,12 +1278,10 @@ int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_
 }
 
 extern "C" size_t omni_moe_gemm2_workspace_bytes(int G, int extra_rows, int64_t M_cap, int H, int I) {
-  if (M_cap < 0 || I <= 0 || H <= 0 || G < 0) return 0;
-  Plan p = make_plan<2>((int)M_cap, 1, G, extra_rows, I, H, M_cap);
-  return p.tile ? TILE_TAIL_BYTES : 0;
+  return omni_host::gemm2_workspace_bytes(G, extra_rows, M_cap, H, I);
 }
 
-extern "C" void omni_moe_reload_tuning(void) { tuning_store() = read_tuning(); }
+extern "C" void omni_moe_reload_tuning(void) { omni_host::tuning_store() = omni_host::read_tuning(); }
 
 extern "C" int omni_moe_gemm_kernel_name(int kind, int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I,
                                          char* buf, size_t buf_bytes) {

@@ -11,7 +11,6 @@
 // wavefronts above; either way a wavefront has at most four dependent passes.  Larger inputs take a count launch,
 // a one-block scan launch and a scatter launch.
 #include <stdlib.h>
-#include <atomic>
 #include <mutex>
 #include "common.h"
 #include "quant_rows.h"
@@ -19,10 +18,10 @@
 
 namespace {
 
-constexpr int GMAX = 256;        // local experts per call
-constexpr int NB = GMAX + 1;     // buckets incl. the dropped one
-constexpr int CH_MULTI = 1024;   // assignments per block in the multi-block path
-constexpr int CH_SINGLE = 4096;  // largest input of the single-block path
+constexpr int GMAX = omni_host::PERM_GMAX;            // local experts per call
+constexpr int NB = omni_host::PERM_NB;                // buckets incl. the dropped one
+constexpr int CH_MULTI = omni_host::PERM_CH_MULTI;    // assignments per block in the multi-block path
+constexpr int CH_SINGLE = omni_host::PERM_CH_SINGLE;  // largest input of the single-block path
 constexpr int NW_SMALL_MAX_N = 1024;  // up to this many assignments the single block has 4 wavefronts, above 16
 
 struct PermArgs {
@@ -271,27 +270,45 @@ __global__ __launch_bounds__(NW * WAVE) void quant_permute_small(const void* __r
 // barrier, one thread counts in with a device-scope acquire-release add (the release half makes the block's stores
 // visible to the device, the acquire half of the last add makes everybody else's visible to the sorting block).
 // No block waits for another.
-template <int MAXV, int V, int NW>
+// FOLD: the logits come as partial sums of the gate projection (RouteArgs::partials): a routing block takes one
+// token, its four wavefronts add the parts up together and the first one routes (blocks [0, T) route).
+// rows == 0: the tokens are quantised already and the launch has no quantising blocks.
+template <int MAXV, int V, int NW, bool FOLD>
 __global__ __launch_bounds__(NW * WAVE) void route_quant_permute_small(const void* __restrict__ x, int64_t rows,
                                                                        int cols, int8_t* __restrict__ q,
                                                                        float* __restrict__ scale, RouteArgs r,
                                                                        PermArgs a, int* arrive) {
+  static_assert(!FOLD || NW == 4, "the block-wide fold is written for four wavefronts");
   constexpr int RPB = NW / 4;
   __shared__ float red[NW];
   __shared__ int s_last;
-  const int route_blocks = (r.T + NW - 1) / NW;
+  const int route_blocks = FOLD ? r.T : (r.T + NW - 1) / NW;
   if ((int)blockIdx.x >= route_blocks) {
     quant_block_rows<MAXV>(x, ((int64_t)blockIdx.x - route_blocks) * RPB, rows, cols, q, scale, red);
     return;
   }
   const int lane = threadIdx.x & (WAVE - 1);
-  const int t = (int)blockIdx.x * NW + threadIdx.x / WAVE;
-  if (t < r.T) {  // the same for a whole wavefront
-    float s[V], bias[V];
+  if constexpr (FOLD) {
+    __shared__ float s_q[FOLD_MAX_GROUPS][WAVE * V];
+    const int t = (int)blockIdx.x, wv = threadIdx.x / WAVE;
+    float s[V], bias[V], tot[V];
     bool in[V];
     route_load_bias<V>(r, lane, bias);
-    route_load_logits<V>(r, t, lane, s, in);
-    route_token<V>(r, t, lane, s, in, bias);
+#pragma unroll
+    for (int j = 0; j < V; ++j) in[j] = lane * V + j < r.E;
+    if (route_fold_block<V>(r, t, lane, wv, in, tot, s_q)) {
+      route_finish_logits<V>(r, t, lane, in, tot, s);
+      route_token<V>(r, t, lane, s, in, bias);
+    }
+  } else {
+    const int t = (int)blockIdx.x * NW + threadIdx.x / WAVE;
+    if (t < r.T) {  // the same for a whole wavefront
+      float s[V], bias[V];
+      bool in[V];
+      route_load_bias<V>(r, lane, bias);
+      route_load_logits<V>(r, t, lane, s, in);
+      route_token<V>(r, t, lane, s, in, bias);
+    }
   }
   __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores are acknowledged before it meets the block
   __syncthreads();
@@ -409,10 +426,7 @@ int sort_waves(int n) {
 
 extern "C" size_t omni_moe_permute_workspace_bytes(int T, int K, int n_local) {
   (void)n_local;
-  int64_t n = (int64_t)T * K;
-  if (n <= CH_SINGLE) return 256;
-  int64_t nblk = (n + CH_MULTI - 1) / CH_MULTI;
-  return (size_t)((nblk + 1) * NB * sizeof(int32_t));
+  return omni_host::permute_workspace_bytes(T, K);
 }
 
 extern "C" int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, int hi, int idx_mode,
@@ -484,25 +498,36 @@ int omni_quant_permute_fused(const void* x_bf16, int T, int H, int8_t* q, float*
 
 // ---- arrival counters of the kernel that routes, quantises and sorts
 // A file-scope device array, zero when the module is loaded; every GPU holds its own copy at its own address (the
-// array's name is only a host-side handle: the device address is asked for once per device).  Calls take the
-// counters in turn, so calls that overlap on one GPU (other streams) use different ones as long as fewer than
-// ARRIVE_SLOTS of them are in flight; each kernel leaves its counter at zero.
+// array's name is only a host-side handle: the device address is asked for once per device).  Every launch leaves
+// its counter at zero.  Which word a call uses is decided by omni_host::ArriveBook (host_logic.h): eager calls take
+// the first 256 words in turn, a call under stream capture gets a word of its (capture, stream) pair from the
+// rest, and when those are used up the call is told so and runs the launches that need no counter.
 namespace {
-constexpr int ARRIVE_SLOTS = 256;
+constexpr int ARRIVE_SLOTS = omni_host::ArriveBook::TOTAL_SLOTS;
 static __device__ int arrive_counters[ARRIVE_SLOTS];
 constexpr int ARRIVE_MAX_DEVICES = 64;
 int* g_arrive_ptr[ARRIVE_MAX_DEVICES];
+omni_host::ArriveBook g_arrive_book[ARRIVE_MAX_DEVICES];
 std::mutex g_arrive_mutex;
-std::atomic<unsigned> g_arrive_next{0};
 
-int next_arrive_counter(int** out) {
+// OMNI_OK with *out set; 1 when the call is being captured and the capture pool is used up (or the device's
+// array cannot be looked up during a capture): the caller then takes the path without a counter
+int next_arrive_counter(hipStream_t st, int** out) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ARRIVE_MAX_DEVICES)
     OMNI_FAIL(OMNI_E_LAUNCH, "route_quant_permute: no current device (or device index >= %d)", ARRIVE_MAX_DEVICES);
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long capture_id = 0;
+  if (hipStreamGetCaptureInfo(st, &status, &capture_id) != hipSuccess) {
+    (void)hipGetLastError();
+    status = hipStreamCaptureStatusNone;
+  }
+  const bool capturing = status == hipStreamCaptureStatusActive;
   int* base;
   {
     std::lock_guard<std::mutex> lock(g_arrive_mutex);
     if (g_arrive_ptr[dev] == nullptr) {
+      if (capturing) return 1;  // the symbol look-up is not a call to make inside a capture
       void* ptr = nullptr;
       const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(arrive_counters));
       if (e != hipSuccess || ptr == nullptr)
@@ -511,7 +536,10 @@ int next_arrive_counter(int** out) {
     }
     base = g_arrive_ptr[dev];
   }
-  *out = base + g_arrive_next.fetch_add(1, std::memory_order_relaxed) % ARRIVE_SLOTS;
+  // capture ids start at 1; 0 stands for "not captured" in the book
+  const int slot = g_arrive_book[dev].take(capturing ? (capture_id ? capture_id : ~0ull) : 0ull, (uintptr_t)st);
+  if (slot < 0) return 1;
+  *out = base + slot;
   return OMNI_OK;
 }
 }  // namespace
@@ -524,25 +552,36 @@ int omni_route_quant_permute_fused(const OmniRouteParams* rp, const void* x_bf16
                                    int32_t* offsets, int32_t* zero_words, int zero_n, void* stream) {
   const int G = hi - lo;
   const int64_t n = (int64_t)T * K;
-  if (T <= 0 || n > CH_SINGLE || G > GMAX || H % 8 != 0 || H > 8 * 256 * 4) return 1;
-  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((size_t)H * 2) % 16 != 0) return 1;
+  if (T <= 0 || n > CH_SINGLE || G > GMAX) return 1;
+  // x_bf16 == null: the tokens are quantised already, the launch routes and sorts only
+  const int64_t qrows = x_bf16 ? T : 0;
+  if (x_bf16 && (H % 8 != 0 || H > 8 * 256 * 4)) return 1;
+  if (x_bf16 && (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((size_t)H * 2) % 16 != 0)) return 1;
+  const bool fold = rp->partials != nullptr;
+  if (fold) {
+    // a routing block per token, four wavefronts: up to 1024 assignments and 16 groups of partial sums
+    const int n_groups = (rp->n_parts + rp->group_len - 1) / rp->group_len;
+    if (n > NW_SMALL_MAX_N || n_groups > OMNI_FOLD_MAX_GROUPS || rp->group_len > 8) return 1;
+  }
+  hipStream_t st = (hipStream_t)stream;
   int* arrive = nullptr;
-  const int rc = next_arrive_counter(&arrive);
-  if (rc) return rc;
-  RouteArgs r{rp->logits, nullptr, 0, 1, 0, nullptr, 0, rp->bias, T, rp->E, rp->n_group, rp->topk_group, K, rp->score_fn,
-              rp->group_mode, rp->masked_fill_zero, rp->weight_from_c, rp->renorm, rp->scale, rp->eps, rp->topk_w,
-              rp->topk_ids};
+  const int rc = next_arrive_counter(st, &arrive);
+  if (rc) return rc;  // 1: no counter to be had (capture pool used up): the caller launches router and sort apart
+  RouteArgs r{rp->logits, rp->partials, rp->n_parts, rp->group_len, fold ? 1 : 0, rp->logits_out, rp->round_logits_bf16,
+              rp->bias, T, rp->E, rp->n_group, rp->topk_group, K, rp->score_fn, rp->group_mode, rp->masked_fill_zero,
+              rp->weight_from_c, rp->renorm, rp->scale, rp->eps, rp->topk_w, rp->topk_ids};
   PermArgs a{rp->topk_ids, (int)n, T, K, lo, G, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, counts, offsets, nullptr, 0,
              zero_words, zero_words ? zero_n : 0};
-  const int nw = sort_waves((int)n), rpb = nw / 4;
-  dim3 grid((unsigned)((T + nw - 1) / nw + (T + rpb - 1) / rpb)), block(nw * WAVE);
-  hipStream_t st = (hipStream_t)stream;
+  const int nw = fold ? 4 : sort_waves((int)n), rpb = nw / 4;
+  const int route_blocks = fold ? T : (T + nw - 1) / nw;
+  dim3 grid((unsigned)(route_blocks + (qrows + rpb - 1) / rpb)), block(nw * WAVE);
   const int V = (rp->E + 63) / 64;
   const int MV = H <= 8 * 256 ? 1 : (H <= 8 * 256 * 2 ? 2 : 4);
 #define RQP_LAUNCH(MAXV, VV)                                                                                                  \
   do {                                                                                                                        \
-    if (nw == 4) hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 4>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, r, a, arrive); \
-    else hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 16>), grid, block, 0, st, x_bf16, (int64_t)T, H, q, scale, r, a, arrive);       \
+    if (fold) hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 4, true>), grid, block, 0, st, x_bf16, qrows, H, q, scale, r, a, arrive); \
+    else if (nw == 4) hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 4, false>), grid, block, 0, st, x_bf16, qrows, H, q, scale, r, a, arrive); \
+    else hipLaunchKernelGGL((route_quant_permute_small<MAXV, VV, 16, false>), grid, block, 0, st, x_bf16, qrows, H, q, scale, r, a, arrive);       \
   } while (0)
 #define RQP_V(MAXV)                      \
   do {                                   \

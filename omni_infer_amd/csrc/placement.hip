@@ -7,7 +7,7 @@
 // lookup on the ids), :337-343 (record_activation).
 #include "common.h"
 
-#include <vector>
+#include <algorithm>
 
 namespace {
 
@@ -38,55 +38,9 @@ __global__ void __launch_bounds__(256) record_activation_kernel(int64_t* counts,
 extern "C" int omni_placement_tables(const int32_t* pattern, int world, int layers, int experts, int rank,
                                      int devices_per_host, int num_deploy, int32_t* position_to_expert,
                                      int32_t* selector) {
-  if (!pattern || !selector) OMNI_FAIL(OMNI_E_INVALID, "placement_tables: null pointer");
-  if (world < 1 || layers < 1 || experts < 1 || devices_per_host < 1)
-    OMNI_FAIL(OMNI_E_INVALID, "placement_tables: bad sizes world=%d layers=%d experts=%d devices_per_host=%d", world, layers, experts, devices_per_host);
-  if (rank < 0 || rank >= world) OMNI_FAIL(OMNI_E_INVALID, "placement_tables: rank %d outside [0,%d)", rank, world);
-  if (num_deploy < experts || num_deploy % world != 0)
-    OMNI_FAIL(OMNI_E_INVALID, "placement_tables: %d deployed positions for %d experts on %d devices", num_deploy, experts, world);
-  const int per_device = num_deploy / world;
-  // positions: device r owns [r*per_device, (r+1)*per_device); its deployed experts take them in id order
-  std::vector<int32_t> pos((size_t)layers * num_deploy, -1);
-  std::vector<int32_t> copies((size_t)layers * experts, 0);
-  for (int l = 0; l < layers; ++l)
-    for (int r = 0; r < world; ++r) {
-      int local = 0;
-      for (int e = 0; e < experts; ++e) {
-        const int32_t v = pattern[((size_t)r * layers + l) * experts + e];
-        if (v != 0 && v != 1) OMNI_FAIL(OMNI_E_INVALID, "placement_tables: pattern[%d][%d][%d] = %d is neither 0 nor 1", r, l, e, v);
-        if (v == 0) continue;
-        if (local >= per_device)
-          OMNI_FAIL(OMNI_E_INVALID, "placement_tables: device %d deploys more than %d experts in layer %d", r, per_device, l);
-        pos[(size_t)l * num_deploy + (size_t)r * per_device + local] = e;
-        copies[(size_t)l * experts + e]++;
-        ++local;
-      }
-    }
-  // selector: for each logical expert the position this rank sends its tokens to: the copy on the rank itself, else
-  // one of the copies on the rank's host, else one of the others, each set shared out by rank modulo its size
-  const int my_host = rank / devices_per_host;
-  std::vector<int32_t> same, far;
-  for (int l = 0; l < layers; ++l)
-    for (int e = 0; e < experts; ++e) {
-      same.clear();
-      far.clear();
-      int32_t own = -1;
-      for (int p = 0; p < num_deploy; ++p) {
-        if (pos[(size_t)l * num_deploy + p] != e) continue;
-        const int dev = p / per_device;
-        if (dev == rank) { if (own < 0) own = p; }
-        else if (dev / devices_per_host == my_host) same.push_back(p);
-        else far.push_back(p);
-      }
-      int32_t s = 0;  // an expert that is deployed nowhere keeps position 0, as in the reference's zero-filled table
-      if (own >= 0) s = own;
-      else if (!same.empty()) s = same[rank % same.size()];
-      else if (!far.empty()) s = far[rank % far.size()];
-      selector[(size_t)l * experts + e] = s;
-    }
-  if (position_to_expert)
-    for (size_t i = 0; i < pos.size(); ++i) position_to_expert[i] = pos[i];
-  return OMNI_OK;
+  // host code on host arrays (host_logic.h)
+  return omni_host::placement_tables(pattern, world, layers, experts, rank, devices_per_host, num_deploy,
+                                     position_to_expert, selector);
 }
 
 extern "C" int omni_moe_remap_ids(const int32_t* ids, int64_t n, const int32_t* map, int n_map, int32_t* out, void* stream) {

@@ -25,10 +25,7 @@
 
 namespace {
 
-constexpr int GATE_SLICE = 128;  // reduction elements of one fma chain
-constexpr int GATE_GROUP = 8;    // slices added up before the groups are
-
-constexpr int FOLD_MAX_GROUPS = 16;  // groups of partial sums the block-wide fold takes (H <= 16384)
+constexpr int GATE_SLICE = 128;  // reduction elements of one fma chain (GATE_GROUP of them make a group: route_body.h)
 
 template <int V>
 __global__ __launch_bounds__(256) void route_kernel(RouteArgs a) {
@@ -51,71 +48,14 @@ __global__ __launch_bounds__(256) void route_kernel(RouteArgs a) {
     for (int j = 0; j < V; ++j) s[j] = in[j] ? row[lane * V + j] : NEG_INF;
   } else {
     // finish the gate projection: groups of `group_len` parts left to right, then the groups left to right
-    const size_t plane = (size_t)a.T * a.E;
-    const float* p0 = a.partials + (size_t)t * a.E + lane * V;
-    const int n_groups = (a.n_parts + a.group_len - 1) / a.group_len;
-    // sum of group g: its parts are all requested before the first add
-    auto load_group = [&](int g, float (&part)[GATE_GROUP][V]) {
-      const int g0 = g * a.group_len;
-      const int gl = (g < n_groups) ? min(a.group_len, a.n_parts - g0) : 0;
-#pragma unroll
-      for (int u = 0; u < GATE_GROUP; ++u)
-#pragma unroll
-        for (int j = 0; j < V; ++j) part[u][j] = (u < gl && in[j]) ? p0[(size_t)(g0 + u) * plane + j] : 0.0f;
-      return gl;
-    };
-    auto fold_group = [&](const float (&part)[GATE_GROUP][V], int gl, float (&q)[V]) {
-#pragma unroll
-      for (int j = 0; j < V; ++j) q[j] = part[0][j];
-#pragma unroll
-      for (int u = 1; u < GATE_GROUP; ++u)
-        if (u < gl) {
-#pragma unroll
-          for (int j = 0; j < V; ++j) q[j] = q[j] + part[u][j];
-        }
-    };
     float tot[V];
     if (a.fold_block) {
       __shared__ float s_q[FOLD_MAX_GROUPS][WAVE * V];
-      // wavefront wv takes groups wv, wv + 4, ...: two of them are loaded before either is added up
-      for (int base = 0; base < n_groups; base += 8) {
-        float pa[GATE_GROUP][V], pb[GATE_GROUP][V], q[V];
-        const int ga = base + wv, gb = base + 4 + wv;
-        const int la = load_group(ga, pa);
-        const int lb = load_group(gb, pb);
-        if (la > 0) {
-          fold_group(pa, la, q);
-#pragma unroll
-          for (int j = 0; j < V; ++j) s_q[ga][lane * V + j] = q[j];
-        }
-        if (lb > 0) {
-          fold_group(pb, lb, q);
-#pragma unroll
-          for (int j = 0; j < V; ++j) s_q[gb][lane * V + j] = q[j];
-        }
-      }
-      __syncthreads();
-      if (wv != 0) return;
-#pragma unroll
-      for (int j = 0; j < V; ++j) tot[j] = s_q[0][lane * V + j];
-      for (int g = 1; g < n_groups; ++g)
-#pragma unroll
-        for (int j = 0; j < V; ++j) tot[j] = tot[j] + s_q[g][lane * V + j];
+      if (!route_fold_block<V>(a, t, lane, wv, in, tot, s_q)) return;
     } else {
-      for (int g = 0; g < n_groups; ++g) {
-        float part[GATE_GROUP][V], q[V];
-        const int gl = load_group(g, part);
-        fold_group(part, gl, q);
-#pragma unroll
-        for (int j = 0; j < V; ++j) tot[j] = (g == 0) ? q[j] : tot[j] + q[j];
-      }
+      route_fold_wave<V>(a, t, lane, in, tot);
     }
-#pragma unroll
-    for (int j = 0; j < V; ++j) {
-      if (a.round_logits_bf16) tot[j] = round_bf16(tot[j]);
-      s[j] = in[j] ? tot[j] : NEG_INF;
-      if (a.logits_out != nullptr && in[j]) a.logits_out[(size_t)t * a.E + lane * V + j] = tot[j];
-    }
+    route_finish_logits<V>(a, t, lane, in, tot, s);
     if (a.K == 0) return;  // the logits were all that was asked for
   }
   route_token<V>(a, t, lane, s, in, bias);
@@ -420,6 +360,58 @@ int omni_route_check(const char* what, int T, int E, int n_group, int topk_group
   return check_route_args(what, T, E, n_group, topk_group, K, score_fn);
 }
 
+int omni_route_launch(const OmniRouteParams* rp, int T, int K, void* stream) {
+  // few tokens: a block per token adds the parts up with its four wavefronts (the latency of one round of
+  // loads instead of one per group); many tokens: a wavefront per token keeps every wavefront routing
+  const int n_groups = rp->partials ? (rp->n_parts + rp->group_len - 1) / rp->group_len : 0;
+  const int fold_block = (rp->partials && T <= 2048 && n_groups <= FOLD_MAX_GROUPS) ? 1 : 0;
+  RouteArgs a{rp->logits, rp->partials, rp->n_parts, rp->group_len, fold_block, rp->logits_out, rp->round_logits_bf16,
+              rp->bias, T, rp->E, rp->n_group, rp->topk_group, K, rp->score_fn, rp->group_mode, rp->masked_fill_zero,
+              rp->weight_from_c, rp->renorm, rp->scale, rp->eps, rp->topk_w, rp->topk_ids};
+  launch_route(a, (hipStream_t)stream);
+  OMNI_CHECK_LAUNCH("route");
+  return OMNI_OK;
+}
+
+int omni_gate_partials(const void* x, int x_dtype, const void* gate_w, int w_dtype, int T, int H, int E, void* partials,
+                       size_t partials_bytes, int* n_parts, int* group_len, void* stream) {
+  if (!x || !gate_w) OMNI_FAIL(OMNI_E_INVALID, "gate: null pointer");
+  if ((x_dtype != OMNI_DT_BF16 && x_dtype != OMNI_DT_F32) || (w_dtype != OMNI_DT_BF16 && w_dtype != OMNI_DT_F32))
+    OMNI_FAIL(OMNI_E_INVALID, "gate: tokens and gate weights must be bf16 or fp32");
+  if (H % GATE_SLICE != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate: H=%d must be a multiple of %d", H, GATE_SLICE);
+  if (((uintptr_t)x % 16) || ((uintptr_t)gate_w % 16)) OMNI_FAIL(OMNI_E_INVALID, "gate: pointers must be 16-byte aligned");
+  if (E > 512) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate: E=%d > 512", E);
+  const size_t need = omni_moe_gate_route_workspace_bytes(T, H, E);
+  if (!partials || partials_bytes < need) OMNI_FAIL(OMNI_E_WORKSPACE, "gate: workspace %zu < %zu", partials_bytes, need);
+  if ((uintptr_t)partials % 16) OMNI_FAIL(OMNI_E_INVALID, "gate: workspace must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  GateArgs g{};
+  g.x = x; g.w = gate_w; g.T = T; g.H = H; g.E = E;
+  g.slices_per_task = gate_slices_per_task(T, H, E);
+  g.n_parts = (H / GATE_SLICE + g.slices_per_task - 1) / g.slices_per_task;
+  const bool tile = g.slices_per_task == GATE_GROUP && T >= gate_tuning().tile_from;
+  g.n_tt = tile ? (T + GT_TOK - 1) / GT_TOK : (T + 63) / 64;
+  g.n_et = tile ? (E + GT_EXP - 1) / GT_EXP : (E + 31) / 32;
+  g.partials = (float*)partials;
+  const int64_t tasks = (int64_t)g.n_parts * g.n_et * g.n_tt;
+  if (tasks > 0x7fffffffLL) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate: too many tasks");
+  dim3 grid((unsigned)tasks), block(tile ? 256 : 64);
+#define GATE_LAUNCH(KERNEL)                                                                                   \
+  do {                                                                                                        \
+    if (x_dtype == OMNI_DT_BF16 && w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((KERNEL<OMNI_DT_BF16, OMNI_DT_F32>), grid, block, 0, st, g); \
+    else if (x_dtype == OMNI_DT_BF16) hipLaunchKernelGGL((KERNEL<OMNI_DT_BF16, OMNI_DT_BF16>), grid, block, 0, st, g);  \
+    else if (w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((KERNEL<OMNI_DT_F32, OMNI_DT_F32>), grid, block, 0, st, g);     \
+    else hipLaunchKernelGGL((KERNEL<OMNI_DT_F32, OMNI_DT_BF16>), grid, block, 0, st, g);                               \
+  } while (0)
+  if (tile) GATE_LAUNCH(gate_tile_kernel);
+  else GATE_LAUNCH(gate_partial_kernel);
+#undef GATE_LAUNCH
+  OMNI_CHECK_LAUNCH("gate_partial");
+  *n_parts = g.n_parts;
+  *group_len = g.slices_per_task == 1 ? GATE_GROUP : 1;
+  return OMNI_OK;
+}
+
 extern "C" int omni_moe_route(const float* logits, const float* bias, int T, int E, int n_group, int topk_group,
                               int K, int score_fn, int group_mode, int masked_fill_zero, int weight_from_c,
                               int renorm, float scale, float eps, float* topk_w, int32_t* topk_ids, void* stream) {
@@ -428,11 +420,9 @@ extern "C" int omni_moe_route(const float* logits, const float* bias, int T, int
   if (!logits || !topk_w || !topk_ids) OMNI_FAIL(OMNI_E_INVALID, "route: null pointer");
   const int rc = check_route_args("route", T, E, n_group, topk_group, K, score_fn);
   if (rc) return rc;
-  RouteArgs a{logits, nullptr, 0, 1, 0, nullptr, 0, bias, T, E, n_group, topk_group, K, score_fn, group_mode, masked_fill_zero,
-              weight_from_c, renorm, scale, eps, topk_w, topk_ids};
-  launch_route(a, (hipStream_t)stream);
-  OMNI_CHECK_LAUNCH("route");
-  return OMNI_OK;
+  OmniRouteParams rp{logits, bias, E, n_group, topk_group, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm,
+                     scale, eps, topk_w, topk_ids};
+  return omni_route_launch(&rp, T, K, stream);
 }
 
 extern "C" size_t omni_moe_gate_route_workspace_bytes(int T, int H, int E) {
@@ -452,50 +442,16 @@ extern "C" int omni_moe_gate_route(const void* x, int x_dtype, const void* gate_
   if (!x || !gate_w) OMNI_FAIL(OMNI_E_INVALID, "gate_route: null pointer");
   if (K == 0 && !logits_out) OMNI_FAIL(OMNI_E_INVALID, "gate_route: nothing to compute (K = 0 and no logits_out)");
   if (K > 0 && (!topk_w || !topk_ids)) OMNI_FAIL(OMNI_E_INVALID, "gate_route: null pointer");
-  if ((x_dtype != OMNI_DT_BF16 && x_dtype != OMNI_DT_F32) || (w_dtype != OMNI_DT_BF16 && w_dtype != OMNI_DT_F32))
-    OMNI_FAIL(OMNI_E_INVALID, "gate_route: tokens and gate weights must be bf16 or fp32");
-  if (H % GATE_SLICE != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: H=%d must be a multiple of %d", H, GATE_SLICE);
-  if (((uintptr_t)x % 16) || ((uintptr_t)gate_w % 16)) OMNI_FAIL(OMNI_E_INVALID, "gate_route: pointers must be 16-byte aligned");
-  if (E > 512) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: E=%d > 512", E);
   if (K > 0) {
     const int rc = check_route_args("gate_route", T, E, n_group, topk_group, K, score_fn);
     if (rc) return rc;
   }
-  const size_t need = omni_moe_gate_route_workspace_bytes(T, H, E);
-  if (!workspace || ws_bytes < need) OMNI_FAIL(OMNI_E_WORKSPACE, "gate_route: workspace %zu < %zu", ws_bytes, need);
-  if ((uintptr_t)workspace % 16) OMNI_FAIL(OMNI_E_INVALID, "gate_route: workspace must be 16-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
-  GateArgs g{};
-  g.x = x; g.w = gate_w; g.T = T; g.H = H; g.E = E;
-  g.slices_per_task = gate_slices_per_task(T, H, E);
-  g.n_parts = (H / GATE_SLICE + g.slices_per_task - 1) / g.slices_per_task;
-  const bool tile = g.slices_per_task == GATE_GROUP && T >= gate_tuning().tile_from;
-  g.n_tt = tile ? (T + GT_TOK - 1) / GT_TOK : (T + 63) / 64;
-  g.n_et = tile ? (E + GT_EXP - 1) / GT_EXP : (E + 31) / 32;
-  g.partials = (float*)workspace;
-  const int64_t tasks = (int64_t)g.n_parts * g.n_et * g.n_tt;
-  if (tasks > 0x7fffffffLL) OMNI_FAIL(OMNI_E_UNSUPPORTED, "gate_route: too many tasks");
-  dim3 grid((unsigned)tasks), block(tile ? 256 : 64);
-#define GATE_LAUNCH(KERNEL)                                                                                   \
-  do {                                                                                                        \
-    if (x_dtype == OMNI_DT_BF16 && w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((KERNEL<OMNI_DT_BF16, OMNI_DT_F32>), grid, block, 0, st, g); \
-    else if (x_dtype == OMNI_DT_BF16) hipLaunchKernelGGL((KERNEL<OMNI_DT_BF16, OMNI_DT_BF16>), grid, block, 0, st, g);  \
-    else if (w_dtype == OMNI_DT_F32) hipLaunchKernelGGL((KERNEL<OMNI_DT_F32, OMNI_DT_F32>), grid, block, 0, st, g);     \
-    else hipLaunchKernelGGL((KERNEL<OMNI_DT_F32, OMNI_DT_BF16>), grid, block, 0, st, g);                               \
-  } while (0)
-  if (tile) GATE_LAUNCH(gate_tile_kernel);
-  else GATE_LAUNCH(gate_partial_kernel);
-#undef GATE_LAUNCH
-  OMNI_CHECK_LAUNCH("gate_partial");
-  // few tokens: a block per token adds the parts up with its four wavefronts (the latency of one round of
-  // loads instead of one per group); many tokens: a wavefront per token keeps every wavefront routing
-  const int group_len = g.slices_per_task == 1 ? GATE_GROUP : 1;
-  const int n_groups = (g.n_parts + group_len - 1) / group_len;
-  const int fold_block = (T <= 2048 && n_groups <= FOLD_MAX_GROUPS) ? 1 : 0;
-  RouteArgs a{nullptr, g.partials, g.n_parts, group_len, fold_block, logits_out, round_logits_bf16, bias, T, E,
-              n_group, topk_group, K, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm, scale, eps, topk_w,
-              topk_ids};
-  launch_route(a, st);
-  OMNI_CHECK_LAUNCH("gate_route");
-  return OMNI_OK;
+  OmniRouteParams rp{nullptr, bias, E, n_group, topk_group, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm,
+                     scale, eps, topk_w, topk_ids};
+  int rc = omni_gate_partials(x, x_dtype, gate_w, w_dtype, T, H, E, workspace, ws_bytes, &rp.n_parts, &rp.group_len, stream);
+  if (rc) return rc;
+  rp.partials = (const float*)workspace;
+  rp.round_logits_bf16 = round_logits_bf16;
+  rp.logits_out = logits_out;
+  return omni_route_launch(&rp, T, K, stream);
 }

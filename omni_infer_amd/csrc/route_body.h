@@ -168,6 +168,94 @@ __device__ __forceinline__ void route_token(const RouteArgs& a, int t, int lane,
   }
 }
 
+// ---- finishing the gate projection from its partial sums (route.hip describes the order): groups of `group_len`
+// parts are added left to right, then the groups left to right.
+constexpr int GATE_GROUP = 8;        // slices added up before the groups are
+constexpr int FOLD_MAX_GROUPS = OMNI_FOLD_MAX_GROUPS;  // groups of partial sums the block-wide fold takes (H <= 16384)
+
+__device__ __forceinline__ int route_fold_groups(const RouteArgs& a) { return (a.n_parts + a.group_len - 1) / a.group_len; }
+
+// parts of group g of token t for the lane's V experts, all requested before the first add; returns their number
+template <int V>
+__device__ __forceinline__ int route_load_group(const RouteArgs& a, int t, int lane, const bool (&in)[V], int g,
+                                                float (&part)[GATE_GROUP][V]) {
+  const size_t plane = (size_t)a.T * a.E;
+  const float* p0 = a.partials + (size_t)t * a.E + lane * V;
+  const int g0 = g * a.group_len;
+  const int gl = (g < route_fold_groups(a)) ? min(a.group_len, a.n_parts - g0) : 0;
+#pragma unroll
+  for (int u = 0; u < GATE_GROUP; ++u)
+#pragma unroll
+    for (int j = 0; j < V; ++j) part[u][j] = (u < gl && in[j]) ? p0[(size_t)(g0 + u) * plane + j] : 0.0f;
+  return gl;
+}
+template <int V>
+__device__ __forceinline__ void route_fold_group(const float (&part)[GATE_GROUP][V], int gl, float (&q)[V]) {
+#pragma unroll
+  for (int j = 0; j < V; ++j) q[j] = part[0][j];
+#pragma unroll
+  for (int u = 1; u < GATE_GROUP; ++u)
+    if (u < gl) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) q[j] = q[j] + part[u][j];
+    }
+}
+// One wavefront adds up everything of token t (one round of loads per group).
+template <int V>
+__device__ __forceinline__ void route_fold_wave(const RouteArgs& a, int t, int lane, const bool (&in)[V], float (&tot)[V]) {
+  const int n_groups = route_fold_groups(a);
+  for (int g = 0; g < n_groups; ++g) {
+    float part[GATE_GROUP][V], q[V];
+    const int gl = route_load_group<V>(a, t, lane, in, g, part);
+    route_fold_group<V>(part, gl, q);
+#pragma unroll
+    for (int j = 0; j < V; ++j) tot[j] = (g == 0) ? q[j] : tot[j] + q[j];
+  }
+}
+// The four wavefronts of a block add up token t together: wavefront wv takes groups wv, wv + 4, ..., two of them
+// loaded before either is added up, the group sums meet in s_q and wavefront 0 adds them left to right.  All four
+// wavefronts call this (block barrier inside); true for wavefront 0, whose tot[] then holds the sums.
+template <int V>
+__device__ __forceinline__ bool route_fold_block(const RouteArgs& a, int t, int lane, int wv, const bool (&in)[V],
+                                                 float (&tot)[V], float (*s_q)[WAVE * V]) {
+  const int n_groups = route_fold_groups(a);
+  for (int base = 0; base < n_groups; base += 8) {
+    float pa[GATE_GROUP][V], pb[GATE_GROUP][V], q[V];
+    const int ga = base + wv, gb = base + 4 + wv;
+    const int la = route_load_group<V>(a, t, lane, in, ga, pa);
+    const int lb = route_load_group<V>(a, t, lane, in, gb, pb);
+    if (la > 0) {
+      route_fold_group<V>(pa, la, q);
+#pragma unroll
+      for (int j = 0; j < V; ++j) s_q[ga][lane * V + j] = q[j];
+    }
+    if (lb > 0) {
+      route_fold_group<V>(pb, lb, q);
+#pragma unroll
+      for (int j = 0; j < V; ++j) s_q[gb][lane * V + j] = q[j];
+    }
+  }
+  __syncthreads();
+  if (wv != 0) return false;
+#pragma unroll
+  for (int j = 0; j < V; ++j) tot[j] = s_q[0][lane * V + j];
+  for (int g = 1; g < n_groups; ++g)
+#pragma unroll
+    for (int j = 0; j < V; ++j) tot[j] = tot[j] + s_q[g][lane * V + j];
+  return true;
+}
+// The finished sums become the logits the router reads: rounded to bf16 when asked, written out when asked.
+template <int V>
+__device__ __forceinline__ void route_finish_logits(const RouteArgs& a, int t, int lane, const bool (&in)[V],
+                                                    float (&tot)[V], float (&s)[V]) {
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    if (a.round_logits_bf16) tot[j] = round_bf16(tot[j]);
+    s[j] = in[j] ? tot[j] : NEG_INF;
+    if (a.logits_out != nullptr && in[j]) a.logits_out[(size_t)t * a.E + lane * V + j] = tot[j];
+  }
+}
+
 // The lane's V logits of token t from a.logits.
 template <int V>
 __device__ __forceinline__ void route_load_logits(const RouteArgs& a, int t, int lane, float (&s)[V], bool (&in)[V]) {

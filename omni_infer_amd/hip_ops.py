@@ -467,6 +467,61 @@ def moe_w8a8_layer_routed(x: torch.Tensor, x_scale: Optional[torch.Tensor], logi
     return out, topk_w, topk_ids
 
 
+def moe_w8a8_block(x: torch.Tensor, gate_w: torch.Tensor, bias: Optional[torch.Tensor], top_k: int, n_group: int,
+                   topk_group: int, score_fn: str, group_mode: int, masked_fill_zero: bool, weight_from_c: bool,
+                   renorm: bool, scale: float, eps: float, lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale,
+                   shared=None, H: int = 0, I: int = 0, x_int8: Optional[torch.Tensor] = None,
+                   pertoken_scale: Optional[torch.Tensor] = None, round_logits_bf16: bool = False,
+                   workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                   rows_dtype: torch.dtype = torch.float32, topk_w: Optional[torch.Tensor] = None,
+                   topk_ids: Optional[torch.Tensor] = None):
+    """The whole block in one library call: ``self.gate.forward(hidden_states.float())``, ``FusedMoE.select_experts``,
+    the quant method's ``apply`` and the sum with the shared expert (deepseek_moe.py:147-152, 244-263, 303).  The same
+    bits as ``moe_gate_route`` followed by ``moe_w8a8_layer``.  ``x`` [T,H] bf16 (or fp32 together with ``x_int8`` /
+    ``pertoken_scale``, the tokens already quantised).  Returns (out, topk_w, topk_ids)."""
+    _need_gpu(x, gate_w, bias, x_int8, pertoken_scale)
+    if x.dim() != 2 or gate_w.dim() != 2 or x.shape[1] != gate_w.shape[1]:
+        raise ValueError("block: x must be [T, H] and the gate weight [E, H]")
+    if x.dtype not in (torch.bfloat16, torch.float32) or gate_w.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("block: tokens and gate weight must be bf16 or fp32")
+    if (x_int8 is None) != (pertoken_scale is None):
+        raise ValueError("block: quantised tokens and their scales come together")
+    x = x.contiguous()
+    gate_w = gate_w.contiguous()
+    T, E, K, dev = x.shape[0], gate_w.shape[0], int(top_k), x.device
+    if x_int8 is not None:
+        x_int8 = x_int8.contiguous()
+        pertoken_scale = pertoken_scale.float().reshape(-1).contiguous()
+    if bias is not None:
+        bias = bias.float().contiguous()
+        if bias.numel() != E:
+            raise ValueError("bias must have one entry per expert")
+    fn = {"softmax": L.OMNI_SCORE_SOFTMAX, "sigmoid": L.OMNI_SCORE_SIGMOID}.get(score_fn)
+    if fn is None:
+        raise ValueError(f"Unsupported scoring function: {score_fn}")
+    if rows_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("rows_dtype must be torch.float32 or torch.bfloat16")
+    if topk_w is None:
+        topk_w = torch.empty(T, K, dtype=torch.float32, device=dev)
+    if topk_ids is None:
+        topk_ids = torch.empty(T, K, dtype=torch.int32, device=dev)
+    sh = shared if shared is not None else (None, None, None, None)
+    need = L.lib().omni_moe_w8a8_block_workspace_bytes(T, K, hi - lo, H, I, E, int(shared is not None), _DT[rows_dtype])
+    if workspace is None or workspace.numel() < need:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    rc = L.lib().omni_moe_w8a8_block(_ptr(x), _DT[x.dtype], _ptr(x_int8), _ptr(pertoken_scale), _ptr(gate_w),
+                                     _DT[gate_w.dtype], _ptr(bias), E, int(n_group), int(topk_group), fn, int(group_mode),
+                                     int(masked_fill_zero), int(weight_from_c), int(renorm), float(scale), float(eps),
+                                     int(round_logits_bf16), _ptr(topk_w), _ptr(topk_ids), T, K, lo, hi, _ptr(w13_packed),
+                                     _ptr(w13_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(sh[0]), _ptr(sh[1]), _ptr(sh[2]),
+                                     _ptr(sh[3]), H, I, _DT[rows_dtype], _ptr(out), _ptr(workspace), workspace.numel(),
+                                     _stream())
+    L.check(rc, "omni_moe_w8a8_block")
+    return out, topk_w, topk_ids
+
+
 def moe_w8a8_layer_static(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: torch.Tensor, topk_ids: torch.Tensor,
                           lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None, H: int = 0,
                           I: int = 0, out: Optional[torch.Tensor] = None,

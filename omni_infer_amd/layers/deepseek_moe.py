@@ -198,19 +198,40 @@ class DeepseekMoE(nn.Module):
         if isinstance(hidden_states, dict):
             x_int8, pertoken_scale = hidden_states["x_int8"], hidden_states["pertoken_scale"]
             hidden_states = hidden_states["x"]
-        topk_weights, topk_ids = self._route(hidden_states, attn_metadata)
         e = self.experts
         lo = self.global_rank * self._positions_per_rank()
         shared = None
         if self.shared_experts is not None:
             gu, dn = self.shared_experts.gate_up_proj, self.shared_experts.down_proj
             shared = (gu.weight, gu.weight_scale, dn.weight, dn.weight_scale)
-        T, K = topk_ids.shape
-        need = ops.L.lib().omni_moe_w8a8_layer_workspace_bytes(T, K, self.local_expert_num, e.hidden_size,
-                                                               e.intermediate_size_per_partition, int(shared is not None),
-                                                               ops._DT[self.rows_dtype])
+        T, K = hidden_states.shape[0], e.top_k
+        E = self.gate.weight.shape[0]
+        need = ops.L.lib().omni_moe_w8a8_block_workspace_bytes(T, K, self.local_expert_num, e.hidden_size,
+                                                               e.intermediate_size_per_partition, E,
+                                                               int(shared is not None), ops._DT[self.rows_dtype])
         if self._workspace is None or self._workspace.numel() < need:
             self._workspace = torch.empty(need, dtype=torch.uint8, device=hidden_states.device)
+        # The ids the router makes go straight into the experts unless something has to see them first: the
+        # placement planner's remap, the forced balance of best_ep (layer.py:273-299), a routing function only
+        # Python can call, or tokens the library cannot quantise itself.  Then the block is one library call:
+        # gate projection, router, quantisation, sort, both GEMMs, weighted sum.
+        opt = model_extra_config.operator_opt_config
+        routing = FusedMoE.builtin_routing_arguments(
+            e.top_k, e.use_grouped_topk, e.renormalize, e.topk_group, e.num_expert_group, e.custom_routing_function,
+            e.scoring_func, e.e_score_correction_bias, self.routed_scaling_factor)
+        one_call = (routing is not None and e.planner is None and not opt.best_ep and e.hidden_size % 128 == 0 and
+                    (x_int8 is not None or hidden_states.dtype == torch.bfloat16) and
+                    hidden_states.dtype in (torch.bfloat16, torch.float32))
+        if one_call:
+            out, _, _ = ops.moe_w8a8_block(hidden_states, self.gate.weight, lo=lo, hi=lo + self.local_expert_num,
+                                           w13_packed=e.w13_weight, w13_scale=e.w13_weight_scale, w2_packed=e.w2_weight,
+                                           w2_scale=e.w2_weight_scale.float(), shared=shared, H=e.hidden_size,
+                                           I=e.intermediate_size_per_partition, x_int8=x_int8,
+                                           pertoken_scale=pertoken_scale,
+                                           round_logits_bf16=self.gate.weight.dtype == torch.bfloat16,
+                                           workspace=self._workspace, rows_dtype=self.rows_dtype, **routing)
+            return out
+        topk_weights, topk_ids = self._route(hidden_states, attn_metadata)
         x_in = hidden_states if x_int8 is None else x_int8
         return ops.moe_w8a8_layer(x_in, pertoken_scale, topk_weights, topk_ids, lo, lo + self.local_expert_num,
                                   e.w13_weight, e.w13_weight_scale, e.w2_weight, e.w2_weight_scale.float(), shared,

@@ -128,6 +128,38 @@ class FusedMoE(torch.nn.Module):
         return topk_weights, topk_ids, row_idx
 
     @staticmethod
+    def builtin_routing_arguments(top_k: int, use_grouped_topk: bool, renormalize: bool, topk_group: Optional[int],
+                                  num_expert_group: Optional[int], custom_routing_function: Optional[Callable],
+                                  scoring_func: str, e_score_correction_bias: Optional[torch.Tensor],
+                                  routed_scaling_factor: Optional[float]):
+        """The arguments the library's router takes for the routing ``select_experts`` (layer.py:301-365) would do,
+        scaling factor included, as keywords of ``hip_ops.moe_w8a8_block`` / ``moe_w8a8_layer_routed``; None for
+        a custom routing function (which only Python can call)."""
+        L = ops.L
+        if custom_routing_function is not None and not use_grouped_topk:
+            return None
+        if use_grouped_topk:
+            if topk_group is None:
+                raise ValueError("Unsupported topk_group is None")
+            if num_expert_group is None:
+                raise ValueError("Unsupported num_expert_group is None")
+            if e_score_correction_bias is None:
+                if scoring_func not in ("softmax", "sigmoid"):
+                    raise ValueError(f"Unsupported scoring function: {scoring_func}")
+                # grouped_topk (fused_moe.py:38-84) times the scaling factor (layer.py:339): the router's last
+                # operation is that multiplication
+                return dict(bias=None, top_k=top_k, n_group=num_expert_group, topk_group=topk_group, score_fn=scoring_func,
+                            group_mode=L.OMNI_GROUP_MAX, masked_fill_zero=True, weight_from_c=True,
+                            renorm=bool(renormalize), scale=float(routed_scaling_factor), eps=0.0)
+            # npu_moe_gating_top_k as called at layer.py:341-351
+            return dict(bias=e_score_correction_bias, top_k=top_k, n_group=num_expert_group, topk_group=topk_group,
+                        score_fn="sigmoid", group_mode=L.OMNI_GROUP_TOP2SUM, masked_fill_zero=False, weight_from_c=False,
+                        renorm=True, scale=float(routed_scaling_factor), eps=float(1e-20))
+        # fused_topk (fused_moe.py:24-34)
+        return dict(bias=None, top_k=top_k, n_group=1, topk_group=1, score_fn="softmax", group_mode=L.OMNI_GROUP_MAX,
+                    masked_fill_zero=False, weight_from_c=False, renorm=bool(renormalize), scale=1.0, eps=0.0)
+
+    @staticmethod
     def gate_and_select_experts(hidden_states: torch.Tensor, gate_weight: torch.Tensor, top_k: int,
                                 use_grouped_topk: bool, renormalize: bool, topk_group: Optional[int] = None,
                                 num_expert_group: Optional[int] = None,

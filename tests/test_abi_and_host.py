@@ -21,10 +21,22 @@ def lib():
     return _lib.lib()
 
 
-def _header_functions():
-    text = open(os.path.join(ROOT, "include", "omni_moe_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(omni_[a-z0-9_]+)\s*\(", text)))
+def _header_functions(names=("omni_moe_hip.h", "omni_moe_diag.h")):
+    found = set()
+    for name in names:
+        text = open(os.path.join(ROOT, "include", name)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        found |= set(re.findall(r"\b(omni_[a-z0-9_]+)\s*\(", text))
+    return sorted(found)
+
+
+def test_operator_header_lists_operators_only():
+    """Measurement helpers live in their own header."""
+    ops_only = _header_functions(("omni_moe_hip.h",))
+    assert not [n for n in ops_only if n.startswith("omni_diag_") or n in ("omni_moe_reload_tuning", "omni_moe_gemm_kernel_name")]
+    assert set(_header_functions(("omni_moe_diag.h",))) == {
+        "omni_diag_mfma_i8_rate", "omni_diag_mfma_i8_tile_rate", "omni_diag_hbm_read_rate", "omni_moe_reload_tuning",
+        "omni_moe_gemm_kernel_name"}
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -35,7 +47,7 @@ def test_library_exports_every_declared_symbol(lib):
         assert hasattr(lib, n), f"{n} declared in the header but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.omni_moe_abi_version() == _lib.ABI_VERSION == 6
+    assert lib.omni_moe_abi_version() == _lib.ABI_VERSION == 7
 
 
 def test_header_constants_match_binding():

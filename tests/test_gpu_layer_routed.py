@@ -287,3 +287,117 @@ def test_routed_entry_when_nothing_is_local_and_when_there_are_no_tokens():
                                             w13_scale=d["s13"], w2_packed=d["w2"], w2_scale=d["s2"], shared=shared,
                                             H=H, I=I, **ra)
     assert tuple(out.shape) == (0, H) and tuple(ids.shape) == (0, 8)
+
+
+# ----------------------------------------------------------------------------- the whole block in one call
+def _block_both(x, gate_w, bias, ra, lo, n, d, shared, H, I, rows_dtype=torch.float32, quantised=False):
+    """gate + router (one call) followed by the layer (one call), against the block entry."""
+    from omni_infer_amd import hip_ops as ops
+    bf16_gate = gate_w.dtype == torch.bfloat16
+    w, ids, _ = ops.moe_gate_route(x, gate_w, bias, ra["top_k"], ra["n_group"], ra["topk_group"], ra["score_fn"],
+                                   ra["group_mode"], ra["masked_fill_zero"], ra["weight_from_c"], ra["renorm"], ra["scale"],
+                                   ra["eps"], round_logits_bf16=bf16_gate)
+    xq = xs = None
+    if quantised:
+        xq, xs = ops.npu_dynamic_quant(x)
+    want = ops.moe_w8a8_layer(xq if quantised else x, xs, w, ids, lo, lo + n, d["w13"], d["s13"], d["w2"], d["s2"], shared,
+                              H=H, I=I, rows_dtype=rows_dtype)
+    got, gw, gids = ops.moe_w8a8_block(x, gate_w, bias, lo=lo, hi=lo + n, w13_packed=d["w13"], w13_scale=d["s13"],
+                                       w2_packed=d["w2"], w2_scale=d["s2"], shared=shared, H=H, I=I, x_int8=xq,
+                                       pertoken_scale=xs, round_logits_bf16=bf16_gate, rows_dtype=rows_dtype, **ra)
+    torch.cuda.synchronize()
+    return (want, w, ids), (got, gw, gids)
+
+
+@pytest.mark.parametrize("T", [1, 5, 64, 128, 200])
+@pytest.mark.parametrize("quantised", [False, True])
+def test_block_entry_matches_gate_route_then_layer(T, quantised):
+    """E=256 in 8 groups, top 8, 32 local experts from id 64, H=1024: up to 128 tokens the launch behind the gate's
+    partial sums adds them up, routes, quantises and sorts; 200 tokens (1600 assignments) take the separate
+    launches.  With tokens that arrive quantised that launch has no quantising blocks."""
+    E, n, H, I, lo = 256, 32, 1024, 256, 64
+    lay = Layer(n, H, I, seed=501, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(502 + T)
+    ra = _route_args(E, "noaux_tc")
+    gate_w = (torch.randn(E, H, generator=g) * 0.05).cuda()
+    for rep in range(2):
+        x = tokens(T, H, 503 + rep).cuda()
+        bias = (torch.randn(E, generator=g) * 0.1).cuda()
+        a, b = _block_both(x, gate_w, bias, ra, lo, n, d, shared, H, I, quantised=quantised)
+        _same(a, b, f"T={T} quantised={quantised} call {rep}")
+
+
+@pytest.mark.parametrize("case", ["bf16_gate", "softmax_top2", "no_shared_bf16_rows", "wide_H"])
+def test_block_entry_variants(case):
+    from omni_infer_amd import _lib as L
+    E, n, H, I, lo, T = 64, 16, 512, 256, 8, 48
+    shared_on, rows_dtype, gdt = True, torch.float32, torch.float32
+    ra = dict(top_k=8, n_group=8, topk_group=4, score_fn="sigmoid", group_mode=L.OMNI_GROUP_TOP2SUM,
+              masked_fill_zero=False, weight_from_c=False, renorm=True, scale=2.5, eps=1e-20)
+    if case == "bf16_gate":
+        gdt = torch.bfloat16
+    elif case == "softmax_top2":
+        E, n, lo = 8, 8, 0
+        ra = _route_args(E, "softmax")
+    elif case == "no_shared_bf16_rows":
+        shared_on, rows_dtype = False, torch.bfloat16
+    elif case == "wide_H":
+        H = 7168          # 56 slices of the gate projection: 7 groups of partial sums
+    lay = Layer(n, H, I, seed=511, shared=shared_on)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]) if shared_on else None
+    g = gen(512)
+    gate_w = (torch.randn(E, H, generator=g) * 0.05).to(gdt).cuda()
+    bias = (torch.randn(E, generator=g) * 0.1).cuda() if ra["score_fn"] == "sigmoid" else None
+    x = tokens(T, H, 513).cuda()
+    a, b = _block_both(x, gate_w, bias, ra, lo, n, d, shared, H, I, rows_dtype=rows_dtype)
+    _same(a, b, case)
+
+
+def test_block_entry_under_graph_capture_and_replay():
+    """The block entry recorded into a HIP graph (its arrival counter then comes from the pool that eager calls
+    never use) and replayed with eager calls of the routed entry in between: every replay gives the eager bits."""
+    from omni_infer_amd import hip_ops as ops
+    E, n, H, I, lo, T = 256, 32, 1024, 256, 0, 24
+    lay = Layer(n, H, I, seed=521, shared=True)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    g = gen(522)
+    ra = _route_args(E, "noaux_tc")
+    gate_w = (torch.randn(E, H, generator=g) * 0.05).cuda()
+    bias = (torch.randn(E, generator=g) * 0.1).cuda()
+    x = tokens(T, H, 523).cuda()
+    K = ra["top_k"]
+    need = ops.L.lib().omni_moe_w8a8_block_workspace_bytes(T, K, n, H, I, E, 1, ops.L.OMNI_DT_F32)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out = torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
+    tw = torch.empty(T, K, dtype=torch.float32, device="cuda")
+    ti = torch.empty(T, K, dtype=torch.int32, device="cuda")
+
+    def call():
+        ops.moe_w8a8_block(x, gate_w, bias, lo=lo, hi=lo + n, w13_packed=d["w13"], w13_scale=d["s13"], w2_packed=d["w2"],
+                           w2_scale=d["s2"], shared=shared, H=H, I=I, workspace=ws, out=out, topk_w=tw, topk_ids=ti, **ra)
+    call()
+    torch.cuda.synchronize()
+    want, want_ids = out.clone(), ti.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call()
+            call()
+    torch.cuda.current_stream().wait_stream(side)
+    logits = torch.randn(T, E, generator=g).cuda()
+    for rep in range(5):
+        out.zero_()
+        ti.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(ti, want_ids), f"replay {rep}"
+        # eager work between the replays, through the counters of the eager pool
+        ops.moe_w8a8_layer_routed(x, None, logits, bias, lo=lo, hi=lo + n, w13_packed=d["w13"], w13_scale=d["s13"],
+                                  w2_packed=d["w2"], w2_scale=d["s2"], shared=shared, H=H, I=I, **ra)
+        torch.cuda.synchronize()

@@ -145,3 +145,114 @@ def test_block_loaded_from_checkpoint_matches_oracle(tmp_path):
         assert torch.equal(out.float().cpu(), out_ref.float())
     finally:
         distributed.set_virtual_ep(1, 0)
+
+
+# ----------------------------------------------------------------------------- the checkpoint's quant description
+def _quant_description(num_bits=None, ignore=("lm_head",), weights=None, inputs=None, fmt="int-quantized"):
+    """A ``quant_model_description.json`` in the layout ``AscendCompressedTensorsConfig.from_config`` parses
+    (compressed_tensors.py:183-222): one config group for every ``Linear``, the weights' ``num_bits`` per module."""
+    if num_bits is None:
+        num_bits = {"self_attn.kv_a_proj_with_mqa": 8, "self_attn.q_a_proj": 8, "mlp.experts": 8, "mlp.shared_experts": 8,
+                    "mlp.gate_up_proj": 8, "mlp.down_proj": 8}
+    w = {"dynamic": False, "num_bits": num_bits, "strategy": "channel", "symmetric": True, "type": "int",
+         "group_size": None}
+    a = {"dynamic": True, "num_bits": 8, "strategy": "token", "symmetric": True, "type": "int", "group_size": None}
+    w.update(weights or {})
+    a.update(inputs or {})
+    return {"config_groups": {"group_0": {"input_activations": a, "output_activations": None, "targets": ["Linear"],
+                                          "weights": w}},
+            "format": fmt, "ignore": list(ignore), "quant_method": "compressed-tensors", "kv_cache_scheme": None,
+            "fa_quant_type": None}
+
+
+def test_quant_config_from_description(tmp_path):
+    import json
+    from omni_infer_amd.layers.linear import ReplicatedLinear
+    from omni_infer_amd.quantization.compressed_tensors import AscendCompressedTensorsConfig as Cfg
+    from omni_infer_amd.quantization.compressed_tensors_moe import AscendCompressedTensorsW8A8Int8MoEMethod
+    from omni_infer_amd.quantization.compressed_tensors_w8a8_int8 import AscendCompressedTensorsW8A8Int8LinearMethod
+    assert Cfg.get_config_filenames() == ["quant_model_description.json"]
+    with pytest.raises(ValueError, match="quant_model_description.json"):
+        Cfg.from_checkpoint_dir(str(tmp_path))
+    (tmp_path / "quant_model_description.json").write_text(json.dumps(_quant_description(ignore=["lm_head", "re:.*mlp\\.gate$"])))
+    cfg = Cfg.from_checkpoint_dir(str(tmp_path))
+    assert list(cfg.target_scheme_map) == ["Linear"] and cfg.quant_format == "int-quantized"
+    assert isinstance(cfg.target_scheme_map["Linear"]["weights"].num_bits, dict)       # kept as written
+    # scheme selection: per-module bits looked up by the layer's name
+    method, bits = cfg.get_moe_method("model.layers.3.mlp.experts")
+    assert isinstance(method, AscendCompressedTensorsW8A8Int8MoEMethod) and bits == 8
+    lin = ReplicatedLinear(128, 64, bias=False, quant_config=None, prefix="x")
+    assert isinstance(cfg.get_quant_method(lin, "model.layers.3.mlp.shared_experts.down_proj"),
+                      AscendCompressedTensorsW8A8Int8LinearMethod)
+    assert cfg.get_quant_method(lin, "model.layers.3.mlp.gate") is None                  # regex entry of ignore
+    assert cfg.get_quant_method(lin, "lm_head") is None                                  # exact entry
+    assert cfg.get_quant_method(torch.nn.ReLU(), "model.layers.3.act") is None           # neither linear nor MoE
+    with pytest.raises(ValueError, match="weight name mismatch"):                        # a module the dict does not name
+        cfg.get_quant_method(lin, "model.layers.3.self_attn.o_proj")
+    # anything but dynamic per-token W8A8 is refused where the reference refuses it
+    for bad in (dict(weights={"symmetric": False}), dict(inputs={"dynamic": False}), dict(inputs={"strategy": "tensor"}),
+                dict(weights={"dynamic": True}), dict(fmt="pack-quantized"), dict(num_bits=16)):
+        c = Cfg.from_config(_quant_description(**bad))
+        with pytest.raises(NotImplementedError):
+            c.get_quant_method(lin, "model.layers.3.mlp.shared_experts.down_proj")
+    c4 = Cfg.from_config(_quant_description(num_bits={"mlp.experts": 4, "mlp.shared_experts": 8}))
+    m4, b4 = c4.get_moe_method("model.layers.3.mlp.experts")
+    assert b4 == 4 and type(m4).__name__ == "AscendCompressedTensorsW4A8Int8MoEMethod"  # empty upstream as well
+    with pytest.raises(RuntimeError, match="Unsupported FusedMoe scheme"):
+        Cfg.from_config(_quant_description(num_bits=16)).get_moe_method("model.layers.3.mlp.experts")
+    # targets: a full layer name and a regex come before the class-name match
+    d = _quant_description()
+    d["config_groups"]["group_1"] = dict(d["config_groups"]["group_0"], targets=["re:.*down_proj$"],
+                                         input_activations=dict(d["config_groups"]["group_0"]["input_activations"], dynamic=False))
+    c = Cfg.from_config(d)
+    with pytest.raises(NotImplementedError):                                             # the regex group is static
+        c.get_quant_method(lin, "model.layers.3.mlp.shared_experts.down_proj")
+    assert c.get_quant_method(lin, "model.layers.3.mlp.shared_experts.gate_up_proj") is not None
+    # the keyword form used in code keeps meaning the built scheme, and refuses others at once
+    assert Cfg(ignore=["gate"]).get_moe_method("x")[1] == 8
+    with pytest.raises(NotImplementedError):
+        Cfg(num_bits=4)
+    with pytest.raises(NotImplementedError):
+        Cfg(dynamic=False)
+
+
+@pytest.mark.gpu
+def test_block_configured_and_loaded_from_a_checkpoint_directory(tmp_path):
+    """A checkpoint directory as it ships: ``quant_model_description.json`` next to the safetensors shards.  The
+    description configures the block (the gate is in ``ignore``), the loader fills it, the forward matches the
+    oracle bit for bit."""
+    import json
+    from oracle import moe_oracle as O
+    from omni_infer_amd import config, distributed
+    from omni_infer_amd.layers.deepseek_moe import DeepseekMoE
+    from omni_infer_amd.loader import iter_safetensors, load_moe_block
+    from omni_infer_amd.quantization.compressed_tensors import AscendCompressedTensorsConfig
+    from tests.helpers import tokens
+    E, H, I, K = 8, 1024, 512, 2
+    config.update_model_extra_config(enable_moe_expert_parallel=True, moe_dispatch_combine=False,
+                                     prefill_dispatch_combine=False)
+    distributed.set_virtual_ep(2, 0)          # experts 0..3 are local
+    try:
+        lay, t, paths = _write_checkpoint(tmp_path, "model.layers.5.mlp", E, H, I, seed=19)
+        (tmp_path / "quant_model_description.json").write_text(json.dumps(_quant_description(ignore=["lm_head", "gate"])))
+        qc = AscendCompressedTensorsConfig.from_checkpoint_dir(str(tmp_path))
+        mc = types.SimpleNamespace(hidden_size=H, n_routed_experts=E, num_experts_per_tok=K, moe_intermediate_size=I,
+                                   n_shared_experts=1, n_group=4, topk_group=2, norm_topk_prob=True, scoring_func="sigmoid",
+                                   topk_method="noaux_tc", routed_scaling_factor=2.5, hidden_act="silu",
+                                   first_k_dense_replace=3)
+        blk = DeepseekMoE(mc, qc, prefix="model.layers.5.mlp", device="cuda")
+        assert blk.experts.num_bits == 8 and blk.gate.quant_method is None
+        load_moe_block(blk, iter_safetensors(paths), "model.layers.5.mlp", E)
+        blk.process_weights_after_loading()
+        x = tokens(40, H, 23)
+        xd = x.cuda()
+        logits = blk.gate(xd.float())[0]
+        bias = t["model.layers.5.mlp.gate.e_score_correction_bias"]
+        bf = lambda v: v.to(torch.bfloat16).float()
+        w_loc = (lay.w1_t[0:4], bf(lay.s13[0:4]), lay.w2_t[0:4], bf(lay.s2[0:4]))
+        shared = (lay.shared[0], bf(lay.sh_s13), lay.shared[2], bf(lay.sh_s2))
+        out_ref = O.deepseek_moe_forward(x, logits.cpu(), bias, w_loc, shared, K, 4, 2, 2.5, (0, 4))
+        out, _ = blk(xd, None, None, 5)
+        assert torch.equal(out.float().cpu(), out_ref.float())
+    finally:
+        distributed.set_virtual_ep(1, 0)
