@@ -161,6 +161,14 @@ int omni_moe_permute(const int32_t* topk_ids, int T, int K, int lo, int hi, int 
 size_t omni_moe_permute_workspace_bytes(int T, int K, int n_local);
 
 /*
+ * Row offsets of the groups from their sizes: offsets[0] = 0, offsets[g+1] = offsets[g] + counts[g].  The grouped
+ * GEMM entries below take offsets; the reference hands its operators the sizes themselves
+ * (`group_list=expert_tokens, group_list_type=1`, fused_moe.py:531-536, :552-574, :670-685) and they add them up
+ * inside.  counts: int32 or int64 (counts_are_int64), G <= 256.
+ */
+int omni_moe_group_offsets(const void* counts, int counts_are_int64, int G, int32_t* offsets, void* stream);
+
+/*
  * Materialise the sorted rows (the expanded_x / dynamic_quant_scale outputs of
  * npu_moe_init_routing(_v2), fused_moe.py:514-515).  row m < offsets[n_local] is a copy of
  * source row token(sorted_src[m]); elem_bytes is the byte size of a row element.
@@ -189,7 +197,9 @@ int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N
  *   Row m of a regular group reads x_q[sorted_src[m] / K] (idx_mode TOKEN_MAJOR) or
  *   x_q[sorted_src[m] % T] (K_MAJOR); sorted_src NULL: row m reads x_q[m].
  *   acc = x_q[row] . W13[g]  (int32, exact);  d = (float(acc) * w13_scale[g][n]) * x_scale[row];
- *   y = silu(d[:I]) * d[I:];  h_scale[m] = max|y| / 127;  h_q = rint(y / h_scale).
+ *   y = silu(d[:I]) * d[I:];  y *= quant_scale[g][n] when quant_scale is given ([G][I] fp32, the smooth_scale of
+ *   fused_experts_w8a8_allgather_ep_a2, fused_moe.py:907; regular groups only);
+ *   h_scale[m] = max|y| / 127;  h_q = rint(y / h_scale).
  *   w13 packed: G matrices of Kdim = H, N = 2I (gate channels first).
  *   acc_dbg (nullable) [M_cap, 2I] receives the int32 accumulators.
  *   workspace: omni_moe_gemm1_workspace_bytes(T, K, G, extra_rows, M_cap, H, I) (same arguments as the call).
@@ -197,8 +207,9 @@ int omni_moe_pack_weight(const int8_t* w, int src_layout, int G, int Kdim, int N
 int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode,
                                 int T, int K, const int8_t* w13_packed, const float* w13_scale,
                                 const int8_t* w13_extra, const float* w13_extra_scale, int extra_rows,
-                                const int32_t* offsets, int G, int H, int I, int64_t M_cap, int flags, int8_t* h_q,
-                                float* h_scale, int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream);
+                                const int32_t* offsets, int G, int H, int I, int64_t M_cap, int flags,
+                                const float* quant_scale, int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
+                                size_t ws_bytes, void* stream);
 size_t omni_moe_gemm1_workspace_bytes(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I);
 
 /*
@@ -270,13 +281,15 @@ int omni_moe_combine(const void* rows, int rows_dtype, const float* topk_w, cons
  *   OMNI_DT_BF16 every row is rounded to bf16 first: the numerics of a bf16 npu_grouped_matmul followed by
  *                npu_moe_finalize_routing (fused_moe.py:570-574 + deepseek_moe.py:292-301); half the bytes.
  *   The same value must be given to omni_moe_w8a8_layer_workspace_bytes.
+ *   quant_scale (nullable, [hi-lo][I] fp32): as for omni_moe_gemm1_swiglu_quant; with it the call is
+ *   fused_experts_w8a8_allgather_ep_a2 (fused_moe.py:844-937) in its default form.
  */
 int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_scale_in, const float* topk_w,
                         const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
                         const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
                         const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
-                        const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16, void* workspace,
-                        size_t ws_bytes, void* stream);
+                        const float* sh2_scale, const float* quant_scale, int H, int I, int rows_dtype, void* out_bf16,
+                        void* workspace, size_t ws_bytes, void* stream);
 size_t omni_moe_w8a8_layer_workspace_bytes(int T, int K, int n_local, int H, int I, int with_shared, int rows_dtype);
 
 /*

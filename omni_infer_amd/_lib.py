@@ -25,9 +25,10 @@ SIGNATURES = {
     "omni_add_rms_norm_quant": (I, [P, P, P, c_int64, I, c_float, P, P, P, P, P]),
     "omni_moe_permute": (I, [P, I, I, I, I, I, P, P, P, P, P, c_size_t, P]),
     "omni_moe_permute_workspace_bytes": (c_size_t, [I, I, I]),
+    "omni_moe_group_offsets": (I, [P, I, I, P, P]),
     "omni_moe_gather_rows": (I, [P, I, I, P, P, P, I, I, I, I, P, P, P]),
     "omni_moe_pack_weight": (I, [P, I, I, I, I, P, P]),
-    "omni_moe_gemm1_swiglu_quant": (I, [P, P, P, I, I, I, P, P, P, P, I, P, I, I, I, c_int64, I, P, P, P, P, c_size_t, P]),
+    "omni_moe_gemm1_swiglu_quant": (I, [P, P, P, I, I, I, P, P, P, P, I, P, I, I, I, c_int64, I, P, P, P, P, P, c_size_t, P]),
     "omni_moe_gemm1_workspace_bytes": (c_size_t, [I, I, I, I, c_int64, I, I]),
     "omni_moe_gemm2_dequant": (I, [P, P, P, P, P, P, I, P, I, I, I, c_int64, I, P, P, P, c_size_t, P]),
     "omni_moe_gemm2_workspace_bytes": (c_size_t, [I, I, c_int64, I, I]),
@@ -40,7 +41,7 @@ SIGNATURES = {
     "omni_diag_hbm_read_rate": (I, [P, c_size_t, I, P, P]),
     "omni_diag_mfma_i8_tile_rate": (I, [P, c_size_t, I, I, I, P, P]),
     "omni_moe_combine": (I, [P, I, P, P, I, I, I, I, I, P, P, P, P, P]),
-    "omni_moe_w8a8_layer": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
+    "omni_moe_w8a8_layer": (I, [P, I, P, P, P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),
     "omni_moe_w8a8_layer_workspace_bytes": (c_size_t, [I, I, I, I, I, I, I]),
     "omni_moe_w8a8_layer_routed": (I, [P, I, P, P, P, I, I, I, I, I, I, I, I, c_float, c_float, P, P, I, I, I, I,
                                        P, P, P, P, P, P, P, P, I, I, I, P, P, c_size_t, P]),

@@ -36,6 +36,7 @@ class ModelOperatorOptConfig:
     enable_moe_expert_parallel: bool = True
     opt_w2_scale_cast: bool = False
     pd_seperate_prefill: bool = False
+    prefill_enable_long_seq: bool = False
 
 
 @dataclass

@@ -237,7 +237,7 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
                const OmniRouteParams* route, int T, int K, int lo, int hi, const int8_t* w13_packed,
                const float* w13_scale, const int8_t* w2_packed, const float* w2_scale, const int8_t* sh13_packed,
                const float* sh13_scale, const int8_t* sh2_packed, const float* sh2_scale, int H, int I, int rows_dtype,
-               void* out_bf16, void* workspace, size_t ws_bytes, void* stream) {
+               void* out_bf16, void* workspace, size_t ws_bytes, void* stream, const float* quant_scale = nullptr) {
   if (T < 0 || K <= 0 || hi <= lo || H <= 0 || I <= 0) OMNI_FAIL(OMNI_E_INVALID, "layer: bad sizes");
   if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "layer: rows_dtype %d", rows_dtype);
   if (T == 0) return OMNI_OK;
@@ -304,7 +304,7 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
     if (rc) return rc;
   }
   rc = omni_gemm1_swiglu_quant_impl(xq, xs, sorted_src, OMNI_IDX_TOKEN_MAJOR, T, K, w13_packed, w13_scale, sh13_packed,
-                                    sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, (int8_t*)(ws + L.h_q),
+                                    sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, quant_scale, (int8_t*)(ws + L.h_q),
                                     (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, tail != nullptr, stream);
   if (rc) return rc;
   // The weighted sum rounds the shared expert's row to bf16 before it adds it to the rounded sum of the routed rows,
@@ -330,11 +330,11 @@ extern "C" int omni_moe_w8a8_layer(const void* x, int x_dtype, const float* x_sc
                                    const int32_t* topk_ids, int T, int K, int lo, int hi, const int8_t* w13_packed,
                                    const float* w13_scale, const int8_t* w2_packed, const float* w2_scale,
                                    const int8_t* sh13_packed, const float* sh13_scale, const int8_t* sh2_packed,
-                                   const float* sh2_scale, int H, int I, int rows_dtype, void* out_bf16,
-                                   void* workspace, size_t ws_bytes, void* stream) {
+                                   const float* sh2_scale, const float* quant_scale, int H, int I, int rows_dtype,
+                                   void* out_bf16, void* workspace, size_t ws_bytes, void* stream) {
   return layer_impl(x, x_dtype, x_scale_in, topk_w, topk_ids, nullptr, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
                     w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, workspace,
-                    ws_bytes, stream);
+                    ws_bytes, stream, quant_scale);
 }
 
 extern "C" int omni_moe_w8a8_layer_routed(const void* x, int x_dtype, const float* x_scale_in, const float* logits,
@@ -381,7 +381,6 @@ extern "C" int omni_moe_w8a8_block(const void* x, int x_dtype, const int8_t* x_q
   if ((x_q == nullptr) != (x_scale == nullptr)) OMNI_FAIL(OMNI_E_INVALID, "block: quantised tokens and their scales come together");
   if (x_q == nullptr && x_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_UNSUPPORTED, "block: tokens that are not quantised yet must be bf16");
   if (rows_dtype != OMNI_DT_F32 && rows_dtype != OMNI_DT_BF16) OMNI_FAIL(OMNI_E_INVALID, "block: rows_dtype %d", rows_dtype);
-  if ((uintptr_t)workspace % 256) OMNI_FAIL(OMNI_E_INVALID, "block: workspace must be 256-byte aligned");
   int rc = omni_route_check("block", T, E, n_group, topk_group, K, score_fn);
   if (rc) return rc;
   const int with_shared = sh13_packed != nullptr;
@@ -389,6 +388,7 @@ extern "C" int omni_moe_w8a8_block(const void* x, int x_dtype, const int8_t* x_q
   const size_t gate_bytes = omni_moe_gate_route_workspace_bytes(T, H, E);
   if (gate_bytes == 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "block: the gate projection needs H %% 128 == 0 (H=%d)", H);
   if (ws_bytes < layer_bytes + gate_bytes) OMNI_FAIL(OMNI_E_WORKSPACE, "block: workspace %zu < %zu", ws_bytes, layer_bytes + gate_bytes);
+  if ((uintptr_t)workspace % 256) OMNI_FAIL(OMNI_E_INVALID, "block: workspace must be 256-byte aligned");
   char* gate_ws = (char*)workspace + layer_bytes;
   OmniRouteParams rp{nullptr, bias, E, n_group, topk_group, score_fn, group_mode, masked_fill_zero, weight_from_c, renorm,
                      scale, eps, topk_w, topk_ids};
@@ -451,6 +451,6 @@ extern "C" int omni_moe_w8a8_layer_static(const void* x, int x_dtype, const floa
   // by a kernel of the call itself (the sorting kernel, or a fill kernel in front of the tile launch); everything
   // else is written before it is read
   return omni_moe_w8a8_layer(x, x_dtype, x_scale_in, topk_w, topk_ids, T, K, lo, hi, w13_packed, w13_scale, w2_packed,
-                             w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, H, I, rows_dtype, out_bf16, ptr,
-                             (size_t)OMNI_STATIC_SCRATCH_BYTES, stream);
+                             w2_scale, sh13_packed, sh13_scale, sh2_packed, sh2_scale, nullptr, H, I, rows_dtype, out_bf16,
+                             ptr, (size_t)OMNI_STATIC_SCRATCH_BYTES, stream);
 }

@@ -74,8 +74,8 @@ void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, in
 int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode, int T,
                                  int K, const int8_t* w13_packed, const float* w13_scale, const int8_t* w13_extra,
                                  const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G, int H, int I,
-                                 int64_t M_cap, int flags, int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
-                                 size_t ws_bytes, bool counters_clean, void* stream);
+                                 int64_t M_cap, int flags, const float* quant_scale, int8_t* h_q, float* h_scale,
+                                 int32_t* acc_dbg, void* workspace, size_t ws_bytes, bool counters_clean, void* stream);
 int omni_gemm2_dequant_impl(const int8_t* h_q, const float* h_scale, const int8_t* w2_packed, const float* w2_scale,
                             const int8_t* w2_extra, const float* w2_extra_scale, int extra_rows, const int32_t* offsets,
                             int G, int H, int I, int64_t M_cap, int out_dtype, void* rows_out, int32_t* acc_dbg,

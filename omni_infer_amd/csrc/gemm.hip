@@ -105,6 +105,7 @@ __global__ __launch_bounds__(NTH) void swiglu_quant_rows(GemmArgs a, int8_t* __r
       if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
       float yv = silu_spec(dg) * du;
       if (bf) yv = round_bf16(yv);
+      if (a.smooth != nullptr && g < a.G) yv = yv * a.smooth[(size_t)g * I + n];
       y[i] = yv;
       amax = fmaxf(amax, fabsf(yv));
     }
@@ -574,7 +575,7 @@ template <int KIND, int WN, bool BF>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][2], const float* row_scale,
                                               uint32_t* stage32, int lane, int wave_row0, int mt_count, int wn, int bx,
                                               int row0, int nrows, const float* __restrict__ wsc, int I,
-                                              int bf16_shift) {
+                                              int bf16_shift, const float* __restrict__ smooth_g) {
   constexpr int NBS = 4 * WN;
   constexpr int GS = 2 * WN;
   // ---- epilogue, one 32-row tile at a time
@@ -595,6 +596,11 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
   }
   wsc_g[0] = wsc[ncol[0]];
   wsc_g[1] = wsc[ncol[1]];
+  // GEMM1: the smoothing factor of the lane's channel (the group's row of GemmArgs::smooth), 1 without
+  float sm_g = 1.0f;
+  if constexpr (KIND == 1) {
+    if (smooth_g != nullptr) sm_g = smooth_g[ncol[0]];
+  }
   if (bf16_out) {
     if constexpr (KIND == 2) {
       const int odd = c32 & 1;
@@ -664,6 +670,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs& a, v16i (&acc)[4][
             if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
             float yv = silu_spec(dg) * du;
             if (bf) yv = round_bf16(yv);
+            if (smooth_g != nullptr) yv = yv * sm_g;
             __builtin_nontemporal_store(yv, ytile + (size_t)below * I);  // read once, by the row quantiser
           } else {
 #pragma unroll
@@ -962,8 +969,12 @@ __global__ __launch_bounds__(128 * WN, 2) void gemm_pipe(GemmArgs a) {
   if constexpr (KIND == 2) {
     if (a.extra_rows_bf16 && a.out_dtype == OMNI_DT_F32 && g >= a.G) bf16_shift = a.offsets[a.G];
   }
+  const float* smooth_g = nullptr;
+  if constexpr (KIND == 1) {
+    if (a.smooth != nullptr && g < a.G) smooth_g = a.smooth + (size_t)g * I;
+  }
   tile_epilogue<KIND, WN, BF>(a, acc, row_scale, stage32, lane, wave_row0, c.mt_count, wn, bx, row0, nrows, wsc, I,
-                              bf16_shift);
+                              bf16_shift, smooth_g);
 #endif
 }
 
@@ -1163,11 +1174,12 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
                                            int idx_mode, int T, int K, const int8_t* w13_packed,
                                            const float* w13_scale, const int8_t* w13_extra,
                                            const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G,
-                                           int H, int I, int64_t M_cap, int flags, int8_t* h_q, float* h_scale,
-                                           int32_t* acc_dbg, void* workspace, size_t ws_bytes, void* stream) {
+                                           int H, int I, int64_t M_cap, int flags, const float* quant_scale,
+                                           int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
+                                           size_t ws_bytes, void* stream) {
   return omni_gemm1_swiglu_quant_impl(x_q, x_scale, sorted_src, idx_mode, T, K, w13_packed, w13_scale, w13_extra,
-                                      w13_extra_scale, extra_rows, offsets, G, H, I, M_cap, flags, h_q, h_scale, acc_dbg,
-                                      workspace, ws_bytes, false, stream);
+                                      w13_extra_scale, extra_rows, offsets, G, H, I, M_cap, flags, quant_scale, h_q,
+                                      h_scale, acc_dbg, workspace, ws_bytes, false, stream);
 }
 
 void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, void* gemm1_ws,
@@ -1186,8 +1198,8 @@ void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, in
 int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode, int T,
                                  int K, const int8_t* w13_packed, const float* w13_scale, const int8_t* w13_extra,
                                  const float* w13_extra_scale, int extra_rows, const int32_t* offsets, int G, int H, int I,
-                                 int64_t M_cap, int flags, int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
-                                 size_t ws_bytes, bool counters_clean, void* stream) {
+                                 int64_t M_cap, int flags, const float* quant_scale, int8_t* h_q, float* h_scale,
+                                 int32_t* acc_dbg, void* workspace, size_t ws_bytes, bool counters_clean, void* stream) {
   int rc = check_group_args("gemm1", offsets, G, H, I, M_cap, extra_rows, w13_extra, w13_extra_scale);
   if (rc) return rc;
   if (M_cap == 0) return OMNI_OK;
@@ -1204,6 +1216,9 @@ int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const 
   a.w = w13_packed; a.w_scale = w13_scale; a.w_extra = w13_extra; a.w_extra_scale = w13_extra_scale;
   a.extra_rows = extra_rows; a.offsets = offsets; a.G = G; a.Kdim = H; a.N = 2 * I; a.flags = flags;
   a.acc_dbg = acc_dbg; a.S = p.S; a.M_cap = M_cap;
+  a.smooth = quant_scale;
+  if (quant_scale && (flags & OMNI_GEMM1_BF16_INTERMEDIATE))
+    OMNI_FAIL(OMNI_E_INVALID, "gemm1: quant_scale belongs to the fp32 epilogue (npu_dequant_swiglu_quant), not to the bf16 one");
   if (p.tile) {
     // fused epilogue: y = silu(gate)*up to scratch, then the row quantiser
     float* y = (float*)workspace;

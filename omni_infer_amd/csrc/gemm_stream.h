@@ -20,6 +20,9 @@ struct GemmArgs {
   int Kdim;  // reduction length
   int N;     // output channels of the GEMM: 2I (GEMM1) or H (GEMM2)
   int flags;
+  // GEMM1: the quant_scale of npu_dequant_swiglu_quant, [G][I] fp32, nullable: y is multiplied by it before the row
+  // is quantised (regular groups only; the extra group has none)
+  const float* smooth;
   float* y;            // GEMM1: [M_cap, I]
   void* rows_out;      // GEMM2: [M_cap, N]
   int out_dtype;
@@ -230,6 +233,11 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
       // a single k share: the wavefront holds the gate and the up sums of its channels, so it
       // dequantises and applies SwiGLU here; the row quantiser is left with the maximum and the rounding
       const bool bf = a.flags & OMNI_GEMM1_BF16_INTERMEDIATE;
+      // the smoothing factors of the lane's channels (rare: asked for here, not carried through the k loop)
+      float smv[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        smv[t] = (a.smooth != nullptr && g < a.G) ? a.smooth[(size_t)g * I + strip[2 * t] * 16 + col] : 1.0f;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if (mt < mt_cnt) {
@@ -249,6 +257,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
                 if (bf) { dg = round_bf16(dg); du = round_bf16(du); }
                 float yv = silu_spec(dg) * du;
                 if (bf) yv = round_bf16(yv);
+                if (a.smooth != nullptr) yv = yv * smv[t];
                 a.y[(size_t)(row0 + rbase + i) * I + n] = yv;
               }
             }

@@ -599,6 +599,35 @@ int omni_route_quant_permute_fused(const OmniRouteParams* rp, const void* x_bf16
   return OMNI_OK;
 }
 
+// ---- group offsets from group sizes: one block, a thread per group, the prefix over the lanes of a wavefront
+// with data-parallel moves and over the wavefronts through LDS
+namespace {
+__global__ __launch_bounds__(GMAX) void group_offsets_kernel(const void* __restrict__ counts, int wide, int G,
+                                                            int32_t* __restrict__ offsets) {
+  __shared__ int wave_tot[GMAX / WAVE];
+  const int g = threadIdx.x, lane = g & (WAVE - 1), wv = g / WAVE;
+  int c = 0;
+  if (g < G) c = wide ? (int)((const int64_t*)counts)[g] : ((const int32_t*)counts)[g];
+  const int incl = wave_incl_scan_dpp_i(c);
+  if (lane == WAVE - 1) wave_tot[wv] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int i = 0; i < wv; ++i) base += wave_tot[i];
+  if (g < G) offsets[g + 1] = base + incl;
+  if (g == 0) offsets[0] = 0;
+}
+}  // namespace
+
+extern "C" int omni_moe_group_offsets(const void* counts, int counts_are_int64, int G, int32_t* offsets, void* stream) {
+  if (G < 0) OMNI_FAIL(OMNI_E_INVALID, "group_offsets: bad size G=%d", G);
+  if (G > GMAX) OMNI_FAIL(OMNI_E_UNSUPPORTED, "group_offsets: %d groups > %d", G, GMAX);
+  if (!offsets || (G > 0 && !counts)) OMNI_FAIL(OMNI_E_INVALID, "group_offsets: null pointer");
+  hipLaunchKernelGGL(group_offsets_kernel, dim3(1), dim3(GMAX), 0, (hipStream_t)stream, counts, counts_are_int64 ? 1 : 0, G,
+                     offsets);
+  OMNI_CHECK_LAUNCH("group_offsets");
+  return OMNI_OK;
+}
+
 extern "C" int omni_moe_gather_rows(const void* x, int elem_bytes, int H, const float* x_scale,
                                     const int32_t* sorted_src, const int32_t* offsets, int n_local, int T, int K,
                                     int idx_mode, void* rows_out, float* scale_out, void* stream) {

@@ -255,10 +255,24 @@ def npu_moe_init_routing(x: torch.Tensor, row_idx: torch.Tensor, expert_idx: tor
     return rows, p.src_to_dst, sorted_ids
 
 
+def group_offsets(counts: torch.Tensor) -> torch.Tensor:
+    """int32 [G+1] row offsets of the groups from their sizes (int32 or int64 [G]): what the reference's grouped
+    operators make of ``group_list`` with ``group_list_type=1`` inside (fused_moe.py:531-536)."""
+    _need_gpu(counts)
+    if counts.dtype not in (torch.int32, torch.int64):
+        counts = counts.to(torch.int64)
+    counts = counts.contiguous()
+    G = counts.numel()
+    offsets = torch.empty(G + 1, dtype=torch.int32, device=counts.device)
+    rc = L.lib().omni_moe_group_offsets(_ptr(counts), int(counts.dtype == torch.int64), G, _ptr(offsets), _stream())
+    L.check(rc, "omni_moe_group_offsets")
+    return offsets
+
+
 def npu_moe_compute_expert_tokens(sorted_expert_idx: torch.Tensor, num_experts: int) -> torch.Tensor:
     """Stands in for ``torch_npu.npu_moe_compute_expert_tokens`` (compressed_tensors_moe.py:237):
     cumulative number of rows up to and including each expert."""
-    return torch.cumsum(torch.bincount(sorted_expert_idx.to(torch.int64), minlength=num_experts), 0).to(torch.int32)
+    return group_offsets(torch.bincount(sorted_expert_idx.to(torch.int64), minlength=num_experts))[1:]
 
 
 _DENSE_OFFSETS = {}
@@ -295,12 +309,23 @@ def pack_weight(w: torch.Tensor, src_layout: int) -> torch.Tensor:
 
 
 # ----------------------------------------------------------------------------- GEMMs
+def _quant_scale(quant_scale: Optional[torch.Tensor], G: int, I: int) -> Optional[torch.Tensor]:
+    """The ``quant_scale`` of ``npu_dequant_swiglu_quant`` as the library takes it: contiguous fp32 [G, I]."""
+    if quant_scale is None:
+        return None
+    _need_gpu(quant_scale)
+    if tuple(quant_scale.shape) != (G, I):
+        raise ValueError(f"quant_scale must be [{G}, {I}] (one factor per expert and intermediate channel)")
+    return quant_scale.float().contiguous()
+
+
 def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_src: Optional[torch.Tensor],
                                idx_mode: int, K: int, w13_packed: torch.Tensor, w13_scale: torch.Tensor,
                                offsets: torch.Tensor, H: int, I: int, M_cap: int,
                                extra: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, extra_rows: int = 0,
                                bf16_intermediate: bool = False, want_acc: bool = False, flags: int = 0,
-                               workspace: Optional[torch.Tensor] = None, out=None):
+                               workspace: Optional[torch.Tensor] = None, out=None,
+                               quant_scale: Optional[torch.Tensor] = None):
     """GEMM1 + dequant + SwiGLU + requant: ``npu_grouped_matmul(int32)`` +
     ``npu_dequant_swiglu_quant`` (fused_moe.py:531-534, :670-677).  Returns (h_q, h_scale, acc)."""
     _need_gpu(x_q, x_scale, w13_packed, w13_scale, offsets)
@@ -316,10 +341,11 @@ def grouped_gemm1_swiglu_quant(x_q: torch.Tensor, x_scale: torch.Tensor, sorted_
     ws_bytes = L.lib().omni_moe_gemm1_workspace_bytes(T, K, G, extra_rows, M_cap, H, I)
     ws = workspace if workspace is not None else torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     ew, es = extra if extra is not None else (None, None)
+    quant_scale = _quant_scale(quant_scale, G, I)
     rc = L.lib().omni_moe_gemm1_swiglu_quant(
         _ptr(x_q), _ptr(x_scale), _ptr(sorted_src), idx_mode, T, K, _ptr(w13_packed), _ptr(w13_scale), _ptr(ew),
         _ptr(es), extra_rows, _ptr(offsets), G, H, I, M_cap,
-        flags | (L.OMNI_GEMM1_BF16_INTERMEDIATE if bf16_intermediate else 0),
+        flags | (L.OMNI_GEMM1_BF16_INTERMEDIATE if bf16_intermediate else 0), _ptr(quant_scale),
         _ptr(h_q), _ptr(h_s), _ptr(acc), _ptr(ws), ws_bytes, _stream())
     L.check(rc, "omni_moe_gemm1_swiglu_quant")
     return h_q, h_s, acc
@@ -336,7 +362,8 @@ def grouped_gemm2_dequant(h_q: torch.Tensor, h_scale: torch.Tensor, w2_packed: t
     dev = h_q.device
     M_cap = h_q.shape[0]
     G = offsets.numel() - 1
-    rows = out if out is not None else torch.zeros(M_cap, H, dtype=out_dtype, device=dev)
+    # rows past the kept total are never written and never read by a consumer that goes by the offsets
+    rows = out if out is not None else torch.empty(M_cap, H, dtype=out_dtype, device=dev)
     acc = torch.zeros(M_cap, H, dtype=torch.int32, device=dev) if want_acc else None
     ew, es = extra if extra is not None else (None, None)
     need = L.lib().omni_moe_gemm2_workspace_bytes(G, extra_rows, M_cap, H, I)
@@ -381,7 +408,7 @@ def moe_combine(rows: torch.Tensor, topk_w: torch.Tensor, src_to_dst: torch.Tens
 def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: torch.Tensor, topk_ids: torch.Tensor,
                    lo: int, hi: int, w13_packed, w13_scale, w2_packed, w2_scale, shared=None, H: int = 0, I: int = 0,
                    workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                   rows_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                   rows_dtype: torch.dtype = torch.float32, quant_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The whole local-share layer in one library call (quant if x is bf16, permute, GEMM1
     epilogue, GEMM2, combine), the shared expert carried as an extra group.
 
@@ -405,10 +432,11 @@ def moe_w8a8_layer(x: torch.Tensor, x_scale: Optional[torch.Tensor], topk_w: tor
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     if out is None:
         out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    quant_scale = _quant_scale(quant_scale, hi - lo, I)
     rc = L.lib().omni_moe_w8a8_layer(_ptr(x), x_dtype, _ptr(x_scale), _ptr(topk_w), _ptr(topk_ids), T, K, lo, hi,
                                      _ptr(w13_packed), _ptr(w13_scale), _ptr(w2_packed), _ptr(w2_scale), _ptr(sh[0]),
-                                     _ptr(sh[1]), _ptr(sh[2]), _ptr(sh[3]), H, I, _DT[rows_dtype], _ptr(out),
-                                     _ptr(workspace), workspace.numel(), _stream())
+                                     _ptr(sh[1]), _ptr(sh[2]), _ptr(sh[3]), _ptr(quant_scale), H, I, _DT[rows_dtype],
+                                     _ptr(out), _ptr(workspace), workspace.numel(), _stream())
     L.check(rc, "omni_moe_w8a8_layer")
     return out
 

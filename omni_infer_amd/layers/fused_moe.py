@@ -63,6 +63,43 @@ def fused_experts_w8a8_allgather_ep(hidden_states: torch.Tensor, pertoken_scale:
                               w2_scale.float(), None, H=H, I=I, rows_dtype=rows_dtype)
 
 
+def fused_experts_w8a8_allgather_ep_a2(hidden_states: torch.Tensor, pertoken_scale: torch.Tensor, w1: torch.Tensor,
+                                       w2: torch.Tensor, w1_scale: torch.Tensor, w2_scale: torch.Tensor,
+                                       topk_weights: torch.Tensor, topk_ids: torch.Tensor, n_routed_experts: int,
+                                       is_prefill: bool, max_num_deployed_expert_per_rank: int,
+                                       smooth_scale: torch.Tensor, hidden_size: Optional[int] = None,
+                                       intermediate_size: Optional[int] = None):
+    """fused_moe.py:844-937, the A2 platform's form of the all-gather expert-parallel pipeline: ``smooth_scale``
+    ([E_loc, I] fp32) multiplies the SwiGLU result before the row quantisation (``quant_scale`` of
+    ``npu_dequant_swiglu_quant``, :907), and under ``pd_seperate_prefill`` the tail is a bf16 grouped GEMM followed
+    by ``npu_moe_finalize_routing`` with bf16 routing weights (:909-918) instead of the fused GEMM2 + finalize
+    (:919-927).  ``prefill_enable_long_seq`` (:873-875) trims the materialised sorted rows to the kept total; no
+    sorted copy of the rows is made here (GEMM1 reads the tokens through the permutation), so there is nothing to
+    trim.  The index patch-up of :879-884 only touches entries past the kept total, which nothing reads.
+    Returns bf16 [T,H], or None when the expert-parallel share is the whole model (no else branch, :867)."""
+    expert_parallel_size = get_ep_group().world_size
+    if expert_parallel_size <= 1:
+        return None
+    opt = model_extra_config.operator_opt_config
+    T, H = hidden_states.shape
+    I = w1_scale.shape[-1] // 2
+    lo = get_world_group().rank_in_group * max_num_deployed_expert_per_rank
+    hi = lo + n_routed_experts
+    if not opt.pd_seperate_prefill:
+        return ops.moe_w8a8_layer(hidden_states, pertoken_scale, topk_weights, topk_ids, lo, hi, w1, w1_scale, w2,
+                                  w2_scale.float(), None, H=H, I=I, quant_scale=smooth_scale)
+    # row_idx_type 0 (:868): the sort's index is source -> slot, which is what the finalize step takes
+    K = topk_ids.shape[1]
+    p = ops.moe_permute(topk_ids, lo, hi, L.OMNI_IDX_TOKEN_MAJOR)
+    M = T * K
+    h_q, h_s, _ = ops.grouped_gemm1_swiglu_quant(hidden_states.contiguous(), pertoken_scale.reshape(-1).contiguous(),
+                                                 p.sorted_src, L.OMNI_IDX_TOKEN_MAJOR, K, w1, w1_scale, p.offsets, H, I, M,
+                                                 quant_scale=smooth_scale)
+    rows, _ = ops.grouped_gemm2_dequant(h_q, h_s, w2, w2_scale.to(torch.bfloat16).float().contiguous(), p.offsets, H, I,
+                                        out_dtype=torch.bfloat16)
+    return ops.moe_combine(rows, topk_weights.to(torch.bfloat16), p.src_to_dst, L.OMNI_IDX_TOKEN_MAJOR, L.OMNI_ORDER_K)
+
+
 def moe_expert_quant_farword(sorted_tokens: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w1_scale: torch.Tensor,
                              w2_scale: torch.Tensor, expert_tokens: torch.Tensor, act_dtype, quant_mode,
                              dynamic_scale: Optional[torch.Tensor] = None):
@@ -74,9 +111,7 @@ def moe_expert_quant_farword(sorted_tokens: torch.Tensor, w1: torch.Tensor, w2: 
         sorted_tokens, pertoken_scale = ops.npu_dynamic_quant(sorted_tokens)
     M, H = sorted_tokens.shape
     I = w1_scale.shape[-1] // 2
-    counts = expert_tokens.to(torch.int32)
-    offsets = torch.zeros(counts.numel() + 1, dtype=torch.int32, device=counts.device)
-    offsets[1:] = torch.cumsum(counts, 0)
+    offsets = ops.group_offsets(expert_tokens)
     h_q, h_s, _ = ops.grouped_gemm1_swiglu_quant(sorted_tokens.contiguous(), pertoken_scale.reshape(-1).contiguous(),
                                                  None, 0, 1, w1, w1_scale, offsets, H, I, M)
     if not model_extra_config.operator_opt_config.opt_w2_scale_cast:
@@ -92,9 +127,7 @@ def gmm_expert(x, expert_tokens, w1, w2, w1_scale, w2_scale, dynamic_scale=None,
     h = x.view(-1, hidden)
     M = h.shape[0]
     I = w1_scale.shape[-1] // 2
-    counts = expert_tokens.to(torch.int32)
-    offsets = torch.zeros(counts.numel() + 1, dtype=torch.int32, device=counts.device)
-    offsets[1:] = torch.cumsum(counts, 0)
+    offsets = ops.group_offsets(expert_tokens)
     h_q, h_s, _ = ops.grouped_gemm1_swiglu_quant(h.contiguous(), dynamic_scale.reshape(-1).contiguous(), None, 0, 1,
                                                  w1, w1_scale, offsets, hidden, I, M)
     rows, _ = ops.grouped_gemm2_dequant(h_q, h_s, w2, w2_scale.to(torch.bfloat16).float().contiguous(), offsets,

@@ -30,17 +30,30 @@ class ReplicatedLinear(nn.Module):
 
     def forward(self, x):
         if self.quant_method is None:
-            # the unquantised replicated linear of the MoE path is the gate (deepseek_moe.py:147-152): its
-            # product runs on the fp32 matrix cores in the library's fixed summation order; a bf16 gate
-            # (deepseek_v3_a2.py:607-613) hands back bf16 logits
-            from .. import hip_ops as ops
-            lead = x.shape[:-1]
-            bf16_gate = self.weight.dtype == torch.bfloat16
-            logits = ops.gate_logits(x.reshape(-1, x.shape[-1]), self.weight, round_logits_bf16=bf16_gate)
-            if bf16_gate:
-                logits = logits.to(torch.bfloat16)
-            return logits.view(*lead, self.output_size), None
+            if not x.is_cuda:
+                raise RuntimeError("omni_infer_amd operators run on the GPU only (got a CPU tensor)")
+            if self._gate_shaped(x):
+                # the unquantised replicated linear of the MoE path is the gate (deepseek_moe.py:147-152): its
+                # product runs on the fp32 matrix cores in the library's fixed summation order; a bf16 gate
+                # (deepseek_v3_a2.py:607-613) hands back bf16 logits
+                from .. import hip_ops as ops
+                lead = x.shape[:-1]
+                bf16_gate = self.weight.dtype == torch.bfloat16
+                logits = ops.gate_logits(x.reshape(-1, x.shape[-1]), self.weight, round_logits_bf16=bf16_gate)
+                if bf16_gate:
+                    logits = logits.to(torch.bfloat16)
+                return logits.view(*lead, self.output_size), None
+            # any other unquantised replicated linear (a projection the checkpoint's ``ignore`` list names, fp16
+            # parameters, a width the gate kernel does not take): the plain product of the reference's
+            # unquantised linear method, ``F.linear(x, weight)`` (linear.py:620-638)
+            return torch.nn.functional.linear(x.to(self.weight.dtype), self.weight), None
         return self.quant_method.apply_weights(self, x, None), None
+
+    def _gate_shaped(self, x) -> bool:
+        """What the library's gate projection takes: at most 512 outputs, a reduction length that is a multiple
+        of 128, bf16 or fp32 operands."""
+        return (self.output_size <= 512 and self.input_size % 128 == 0 and
+                x.dtype in (torch.bfloat16, torch.float32) and self.weight.dtype in (torch.bfloat16, torch.float32))
 
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor) -> None:
         """vLLM's ``ReplicatedLinear.weight_loader``: a whole-parameter copy; shapes must agree."""

@@ -18,7 +18,8 @@ from .. import _lib as L
 from .. import hip_ops as ops
 from ..config import model_extra_config
 from ..distributed import get_ep_group
-from ..layers.fused_moe import fused_experts_w8a8_allgather_ep, moe_expert_quant_farword
+from ..layers.fused_moe import (fused_experts_w8a8_allgather_ep, fused_experts_w8a8_allgather_ep_a2,
+                                moe_expert_quant_farword)
 
 SEQ_SPLIT_LENGTH = 4096
 
@@ -106,6 +107,12 @@ class AscendCompressedTensorsW8A8Int8MoEMethod:
                         "Use the all-gather expert-parallel flags (prefill_dispatch_combine=False, "
                         "moe_dispatch_combine=False) for one GPU's share of a larger model.")
                 out = fused_experts_w8a8_one_rank_dispatch_combine(layer, x, topk_weights, topk_ids)
+            elif os.getenv("ASCEND_PLATFORM", "A3") == "A2":   # the reference's own switch (:157)
+                out = fused_experts_w8a8_allgather_ep_a2(
+                    hidden_states=x, pertoken_scale=pertoken_scale, w1=layer.w13_weight, w2=layer.w2_weight,
+                    w1_scale=layer.w13_weight_scale, w2_scale=layer.w2_weight_scale, topk_weights=topk_weights,
+                    topk_ids=topk_ids, n_routed_experts=n_local, is_prefill=is_prefill,
+                    max_num_deployed_expert_per_rank=max_num_deployed_expert_per_rank, smooth_scale=self.smooth_scale)
             else:
                 out = fused_experts_w8a8_allgather_ep(
                     hidden_states=x, pertoken_scale=pertoken_scale, w1=layer.w13_weight, w2=layer.w2_weight,

@@ -51,6 +51,11 @@ tests/test_oracle_pins.py):
   wrong group's scale, a missing per-token scale, swapped halves must fail),
   and the end-to-end dense brute force (every token through every selected
   expert without any permutation).
+* fused_experts_w8a8_allgather_ep_a2 ... permutation-free fp64 brute force with the
+  smoothing factors inside (dropping them, or applying them after the row
+  quantisation instead of before, fails); with factors of one the bits of
+  fused_experts_w8a8_allgather_ep; the bf16 tail against the same brute force
+  within the bf16 bar, and != the fp32-row tail.
 * moe_expert_quant_forward ... permutation-free fp64 witness; its second
   stage within one bf16 step of the fp64 closed form with the w2 scale it was
   asked to use (a skipped bf16 rounding of that scale fails).
@@ -664,6 +669,42 @@ def fused_experts_w8a8_allgather_ep(x_int8, pertoken_scale, w1, w2, w1_scale, w2
         acc2 = grouped_matmul_int32(hq, w2, counts)
         return out, dict(idx=idx, counts=counts, rows=rows, row_scale=scale, acc1=acc1, y=y, h_q=hq, h_s=hs,
                          acc2=acc2, out32=out32)
+    return out
+
+
+def fused_experts_w8a8_allgather_ep_a2(x_int8, pertoken_scale, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids,
+                                       expert_range, smooth_scale, pd_seperate_prefill=False, return_stages=False):
+    """``fused_experts_w8a8_allgather_ep_a2`` (fused_moe.py:844-937): the local-share pipeline of the A2 platform
+    branch.  As ``fused_experts_w8a8_allgather_ep`` with ``quant_scale=smooth_scale`` ([E_loc, I] fp32) inside
+    ``npu_dequant_swiglu_quant`` (:907), and two tails:
+
+    * default (:919-927): ``npu_grouped_matmul_finalize_routing`` on fp32 sums with a zero shared input;
+    * ``pd_seperate_prefill`` (:909-918): ``npu_grouped_matmul(..., output_dtype=bf16)`` with the bf16 ``w2_scale``
+      that ``process_weights_after_loading`` makes under that flag (compressed_tensors_moe.py:100-101), then
+      ``npu_moe_finalize_routing(rows, None, None, None, topk_weights.to(bf16), expanded_x_idx, topk_ids,
+      drop_pad_mode=3)`` with the source-to-slot index that ``row_idx_type=0`` asks of the sort (:868):
+      out[n] = sum_k float(bf16(w[n,k])) * float(rows[slot(n*K+k)]) over the kept assignments, k ascending, fp32,
+      rounded to bf16.  (What mode 3 does with a dropped assignment is not observable here: it contributes nothing.)
+
+    The index patch-up of :879-884 only rewrites entries past the kept total, which nothing reads.
+    """
+    T, K = topk_ids.shape
+    rows, idx, counts, scale = moe_init_routing_v2(x_int8, topk_ids, pertoken_scale, expert_range)
+    acc1 = grouped_matmul_int32(rows, w1, counts)
+    hq, hs, y = dequant_swiglu_quant(acc1, w1_scale, scale, counts, quant_scale=smooth_scale, return_fp32=True)
+    if pd_seperate_prefill:
+        out_rows = grouped_matmul_dequant(hq, w2, w2_scale.to(torch.bfloat16), hs, counts, out_dtype=torch.bfloat16)
+        src_to_dst = torch.full((T * K,), -1, dtype=torch.int32)
+        src_to_dst[idx.to(torch.int64)] = torch.arange(idx.numel(), dtype=torch.int32)
+        out = moe_finalize_routing(out_rows, None, topk_weights.to(torch.bfloat16), src_to_dst, drop_pad_mode=2)
+    else:
+        w_sorted = topk_weights.reshape(-1)[idx.to(torch.int64)]
+        row_index = (idx // K).to(torch.int64)
+        shared_input = torch.zeros(T, w2.shape[2], dtype=torch.bfloat16)
+        out = grouped_matmul_finalize_routing(hq, w2, counts, w2_scale.float(), hs, shared_input, w_sorted, row_index,
+                                              T).to(torch.bfloat16)
+    if return_stages:
+        return out, dict(idx=idx, counts=counts, y=y, h_q=hq, h_s=hs)
     return out
 
 

@@ -75,16 +75,29 @@ def test_argument_validation_returns_codes(lib):
     assert lib.omni_moe_permute(p, 4, 8, 5, 5, 0, p, p, p, p, p, 1 << 20, None) == -1
     assert lib.omni_moe_permute(p, 4096, 8, 0, 32, 0, p, p, p, p, p, 16, None) == -3                    # workspace
     assert lib.omni_moe_pack_weight(p, 0, 1, 100, 16, p, None) == -2                                    # Kdim % 64
-    assert lib.omni_moe_gemm1_swiglu_quant(p, p, None, 0, 4, 1, p, p, None, None, 0, p, 1, 7168, 2000, 4, 0, p, p,
+    assert lib.omni_moe_gemm1_swiglu_quant(p, p, None, 0, 4, 1, p, p, None, None, 0, p, 1, 7168, 2000, 4, 0, None, p, p,
                                            None, p, 1 << 30, None) == -2                                # I % 64
-    assert lib.omni_moe_gemm1_swiglu_quant(p, p, None, 0, 4, 1, p, p, None, None, 0, p, 1, 7168, 2048, 4, 0, p, p,
+    assert lib.omni_moe_gemm1_swiglu_quant(p, p, None, 0, 4, 1, p, p, None, None, 0, p, 1, 7168, 2048, 4, 0, None, p, p,
                                            None, p, 16, None) == -3
+    assert lib.omni_moe_gemm1_swiglu_quant(p, p, None, 0, 4, 1, p, p, None, None, 0, p, 1, 7168, 2048, 4, 1, p, p, p,
+                                           None, p, 1 << 30, None) == -1            # quant_scale with the bf16 epilogue
+    assert lib.omni_moe_group_offsets(p, 0, 300, p, None) == -2                                         # > 256 groups
+    assert lib.omni_moe_group_offsets(None, 0, 4, p, None) == -1
     assert lib.omni_moe_gemm2_dequant(p, p, p, p, None, None, 0, p, 1, 7168, 2048, 4, 5, p, None, None, 0, None) == -1
     assert lib.omni_moe_combine(p, 1, p, p, 0, 0, 4, 100, 64, None, None, None, p, None) == -2          # K > 64
-    assert lib.omni_moe_w8a8_layer(p, -1, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, 1, p,
-                                   p, 1 << 30, None) == -1                                              # int8 w/o scale
-    assert lib.omni_moe_w8a8_layer(p, 0, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, 7168, 2048, 2, p,
-                                   p, 1 << 30, None) == -1                                              # rows_dtype f16
+    assert lib.omni_moe_w8a8_layer(p, -1, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, None, 7168, 2048, 1,
+                                   p, p, 1 << 30, None) == -1                                           # int8 w/o scale
+    assert lib.omni_moe_w8a8_layer(p, 0, None, p, p, 4, 8, 0, 32, p, p, p, p, None, None, None, None, None, 7168, 2048, 2,
+                                   p, p, 1 << 30, None) == -1                                           # rows_dtype f16
+    # the whole block: the gate's and the router's checks come first
+    block = lambda x_dtype, xq, xs, H, E: lib.omni_moe_w8a8_block(
+        p, x_dtype, xq, xs, p, 1, None, E, 8, 4, 1, 1, 0, 0, 1, 2.5, 1e-20, 0, p, p, 4, 8, 0, 32, p, p, p, p, None, None,
+        None, None, H, 2048, 1, p, p, 1 << 30, None)
+    assert block(1, None, None, 7168, 256) == -2 and b"bf16" in lib.omni_moe_last_error()             # fp32 tokens, not quantised
+    assert block(0, p, None, 7168, 256) == -1                                                           # int8 without scales
+    assert block(0, None, None, 7168, 1024) == -2                                                       # E > 512
+    assert block(0, None, None, 7200, 256) == -2 and b"128" in lib.omni_moe_last_error()              # H % 128
+    assert lib.omni_moe_w8a8_block_workspace_bytes(4, 8, 32, 7200, 2048, 256, 1, 1) == 0
     assert lib.omni_moe_w8a8_layer_workspace_bytes(4, 8, 32, 7168, 2048, 1, 2) == 0
     # router and layer in one call: the router's checks come first, then the layer's
     routed = lambda logits, E, n_group, T, rows_dtype: lib.omni_moe_w8a8_layer_routed(

@@ -127,12 +127,46 @@ def test_config3_full_size_prefill(env, dsv3_full, rows_dtype):
         assert r < 5e-3
 
 
-# ------------------------------------------------------------------ config 4 at 4096 tokens
-def test_config4_pangu_4096_tokens(env):
+# ------------------------------------------------------------------ config 4 at its real shape
+@pytest.fixture(scope="module")
+def pangu_full(env):
+    """Pangu-Ultra-MoE widths (H=7680, I=2048), 32 local experts of 256 + shared: the whole token sweep of config 4."""
+    return DeviceLayer(env.ops, 32, 7680, 2048, seed=400)
+
+
+@pytest.mark.parametrize("T", [1, 16, 128, 1024])
+def test_config4_pangu_token_sweep_32_of_256(env, pangu_full, T):
+    """The sweep of config 4 below 4096 tokens at the full 32 local experts of 256: router over all 256 experts
+    with the local range favoured, through the entry that routes and runs the layer in one call (1 to 128 tokens:
+    stream kernels behind the launch that routes, quantises and sorts; 1024 tokens: tile kernels), bit exact."""
+    lay = pangu_full
+    g = gen(410 + T)
+    E, lo = 256, 96
+    x = tokens(T, 7680, 410 + T)
+    logits = torch.randn(T, E, generator=g)
+    logits[:, lo:lo + 32] += 1.5
+    bias = torch.randn(E, generator=g) * 0.01
+    w_ref, id_ref = O.route_noaux_tc(logits, bias, 8, 8, 4, 2.5)
+    w1_t, s13, w2_t, s2, shared = lay.host()
+    xq, xs = O.dynamic_quant(x)
+    ref = O.fused_experts_w8a8_allgather_ep(xq, xs, w1_t, w2_t, s13, s2, w_ref, id_ref, (lo, lo + 32))
+    ref = ref + O.shared_expert_mlp(x, *shared)
+    d = lay.dev
+    out, w, ids = env.ops.moe_w8a8_layer_routed(
+        x.cuda(), None, logits.cuda(), bias.cuda(), top_k=8, n_group=8, topk_group=4, score_fn="sigmoid",
+        group_mode=env.L.OMNI_GROUP_TOP2SUM, masked_fill_zero=False, weight_from_c=False, renorm=True, scale=2.5,
+        eps=1e-20, lo=lo, hi=lo + 32, w13_packed=d["w13"], w13_scale=d["s13"], w2_packed=d["w2"], w2_scale=d["s2"],
+        shared=lay.dev_shared, H=lay.H, I=lay.I)
+    torch.cuda.synchronize()
+    assert torch.equal(ids.cpu(), id_ref) and torch.equal(w.cpu(), w_ref)
+    _check(out, ref, exact=True)
+
+
+def test_config4_pangu_4096_tokens(env, pangu_full):
     """Pangu-Ultra-MoE shape: H=7680, I=2048, 32 local experts of 256, shared expert, 4096 tokens; sigmoid
     grouped top-8 routing over all 256 experts with the local ones favoured (global ids, local range
     filter), router and layer against the oracle."""
-    lay = DeviceLayer(env.ops, 32, 7680, 2048, seed=400)
+    lay = pangu_full
     g = gen(401)
     T, E, lo = 4096, 256, 96
     x = tokens(T, 7680, 401)

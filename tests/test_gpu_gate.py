@@ -129,3 +129,25 @@ def test_gate_argument_errors(ops):
         ops.gate_logits(x, torch.zeros(8, 128, device="cuda"))
     with pytest.raises(ValueError):
         ops.gate_logits(x.to(torch.float16), w)
+
+
+def test_unquantised_replicated_linear_that_is_not_a_gate():
+    """A replicated linear the ``ignore`` list keeps unquantised, with a width the gate kernel does not take (7168
+    outputs), or fp16 parameters: the plain product of the reference's unquantised linear method, not an error."""
+    from omni_infer_amd.layers.linear import ReplicatedLinear
+    from omni_infer_amd.quantization.compressed_tensors import AscendCompressedTensorsConfig
+    cfg = AscendCompressedTensorsConfig(ignore=["down_proj"])
+    g = torch.Generator().manual_seed(5)
+    lin = ReplicatedLinear(2048, 7168, bias=False, quant_config=cfg, params_dtype=torch.bfloat16,
+                           prefix="model.layers.3.mlp.shared_experts.down_proj", device="cuda")
+    assert lin.quant_method is None
+    lin.weight.data.copy_((torch.randn(7168, 2048, generator=g) * 0.02).to(torch.bfloat16))
+    x = torch.randn(5, 2048, generator=g).to(torch.bfloat16).cuda()
+    out, _ = lin(x)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (5, 7168)
+    want = x.float().cpu() @ lin.weight.data.float().cpu().t()
+    assert float((out.float().cpu() - want).norm() / want.norm()) < 1e-2
+    half = ReplicatedLinear(256, 64, bias=False, quant_config=None, params_dtype=torch.float16, prefix="gate", device="cuda")
+    half.weight.data.copy_((torch.randn(64, 256, generator=g) * 0.05).to(torch.float16))
+    out, _ = half(torch.randn(3, 256, generator=g).to(torch.float16).cuda())
+    assert out.dtype == torch.float16 and tuple(out.shape) == (3, 64)

@@ -226,9 +226,7 @@ def test_config4_pangu_shape(env, T):
     logits = blk.gate(x.cuda().float())[0]
     out_ref, st = _block_reference(lay, x, logits.cpu(), bias, lo, 4)
     out, _ = blk(x.cuda(), None, None, 3)
-    # at 1024 tokens the fp32 row buffer would pass 256 MiB, so the rows between GEMM2 and the combine are
-    # bf16 (the numerics of the separate GEMM2 and finalize operators): tolerance instead of bit equality
-    _check_out(out, out_ref, exact=T < 1024)
+    _check_out(out, out_ref, exact=True)   # fp32 rows at every size (the block's default): bit equality
 
 
 # ------------------------------------------------------------------ config 5: skewed load
@@ -356,3 +354,85 @@ def test_layer_call_sequence_is_graph_capturable(env, T):
     torch.cuda.synchronize()
     replayed = out.clone()
     assert torch.equal(step(), replayed), "replay on new inputs differs from the eager run"
+
+
+# ------------------------------------------------------------------ the A2 platform branch of apply()
+@pytest.mark.parametrize("shape", ["config1_toy", "config3_reduced"])
+@pytest.mark.parametrize("pd_seperate_prefill", [False, True])
+def test_apply_a2_platform_branch(env, monkeypatch, shape, pd_seperate_prefill):
+    """``ASCEND_PLATFORM=A2`` sends the all-gather expert-parallel branch of ``apply()`` to
+    ``fused_experts_w8a8_allgather_ep_a2`` (compressed_tensors_moe.py:157-170; fused_moe.py:844-937): smoothing
+    factors inside the dequant-SwiGLU-quant step (other than one here, so that they show), and under
+    ``pd_seperate_prefill`` the bf16 GEMM2 + finalize tail with a bf16 w2 scale.  The toy layer of config 1 as rank 1
+    of 2 (stream kernels) and config 3 reduced to 2 local experts of 16 with outlier channels (tile kernels), bit
+    exact against the oracle's A2 pipeline."""
+    monkeypatch.setenv("ASCEND_PLATFORM", "A2")
+    env.config.update_model_extra_config(enable_moe_expert_parallel=True, moe_dispatch_combine=False,
+                                         prefill_dispatch_combine=False, pd_seperate_prefill=pd_seperate_prefill)
+    try:
+        if shape == "config1_toy":
+            n_local, E, K, H, I, T, ep, rank, out_frac = 4, 8, 2, 1024, 512, 64, 2, 1, 0.0
+        else:
+            n_local, E, K, H, I, T, ep, rank, out_frac = 2, 16, 4, 7168, 2048, 1024, 8, 3, 0.001
+        lay = _bf16_scales(Layer(n_local, H, I, seed=61))
+        m = _make_fused_moe(env, lay, E, K, ep, rank)
+        m.quant_method.process_weights_after_loading(m)
+        assert bool((m.quant_method.smooth_scale == 1).all())          # what the reference makes (:113)
+        g = gen(62)
+        smooth = torch.rand(n_local, I, generator=g) * 1.5 + 0.25
+        m.quant_method.smooth_scale = smooth.cuda()
+        x = tokens(T, H, 63, outlier_frac=out_frac)
+        lo = rank * n_local
+        if shape == "config1_toy":
+            ids = torch.rand(T, E, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+        else:   # every token on both local experts and on two remote ones
+            ids = torch.cat([(torch.rand(T, 2, generator=g).argsort(dim=1) + lo).to(torch.int32),
+                             torch.randint(8, 16, (T, 2), generator=g).to(torch.int32)], dim=1)
+        w = torch.rand(T, K, generator=g)
+        xq, xs = O.dynamic_quant(x)
+        ref = O.fused_experts_w8a8_allgather_ep_a2(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (lo, lo + n_local),
+                                                   smooth, pd_seperate_prefill=pd_seperate_prefill)
+        out = m(xq.cuda(), w.cuda(), ids.cuda(), xs.cuda(), None)
+        _check_out(out, ref)
+        # with the factors the reference ships (ones) the branch gives the bits of the A3 pipeline
+        if not pd_seperate_prefill:
+            m.quant_method.smooth_scale = torch.ones(n_local, I, device="cuda")
+            ref3 = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (lo, lo + n_local))
+            _check_out(m(xq.cuda(), w.cuda(), ids.cuda(), xs.cuda(), None), ref3)
+    finally:
+        env.config.update_model_extra_config(pd_seperate_prefill=False)
+        env.dist.set_virtual_ep(1, 0)
+
+
+def test_gemm1_quant_scale_on_both_kernels_and_split_k(env):
+    """The smoothing factors in every GEMM1 epilogue that exists: the stream kernel that applies SwiGLU itself,
+    its split-k form finished by the row kernel (forced through the tuning variable), and the tile kernel;
+    int8 rows and row scales against the oracle's dequant-SwiGLU-quant with ``quant_scale``."""
+    import os
+    L, ops = env.L, env.ops
+    G, H, I = 3, 1024, 256
+    lay = Layer(G, H, I, seed=71)
+    d = lay.to_device()
+    g = gen(72)
+    smooth = torch.rand(G, I, generator=g) * 1.5 + 0.25
+    for rows_per_group, env_g1 in ((9, None), (9, "1,1,4,2"), (150, None)):
+        counts = torch.tensor([rows_per_group, 0, rows_per_group + 3])
+        M = int(counts.sum())
+        x = tokens(M, H, 73 + rows_per_group)
+        xq, xs = O.dynamic_quant(x)
+        acc = O.grouped_matmul_int32(xq, lay.w1_t, counts)
+        hq_ref, hs_ref = O.dequant_swiglu_quant(acc, lay.s13, xs, counts, quant_scale=smooth)
+        if env_g1:
+            os.environ["OMNI_MOE_G1"] = env_g1
+            L.lib().omni_moe_reload_tuning()
+        try:
+            offsets = ops.group_offsets(counts.cuda())
+            hq, hs, _ = ops.grouped_gemm1_swiglu_quant(xq.cuda(), xs.cuda(), None, 0, 1, d["w13"], d["s13"], offsets, H, I, M,
+                                                       quant_scale=smooth.cuda())
+            torch.cuda.synchronize()
+        finally:
+            if env_g1:
+                del os.environ["OMNI_MOE_G1"]
+                L.lib().omni_moe_reload_tuning()
+        assert torch.equal(hs.cpu(), hs_ref), f"row scales, {rows_per_group} rows per group, G1={env_g1}"
+        assert torch.equal(hq.cpu(), hq_ref), f"int8 rows, {rows_per_group} rows per group, G1={env_g1}"

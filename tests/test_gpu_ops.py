@@ -494,3 +494,20 @@ def test_tile_numbering_row_count_edges(ops, tuning, shared):
     out = ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), 2, 2 + n_local, d["w13"], d["s13"], d["w2"], d["s2"],
                              sh, H=H, I=I)
     _eq(out, want, f"row-count edges shared={shared}")
+
+
+@pytest.mark.parametrize("G", [1, 33, 64, 65, 200, 256])
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+def test_group_offsets(G, dtype):
+    """Row offsets of the groups from their sizes (what the reference's grouped operators make of ``group_list``
+    with ``group_list_type=1``): against numpy's cumulative sum, empty groups included."""
+    import numpy as np
+    from omni_infer_amd import hip_ops as ops
+    g = torch.Generator().manual_seed(900 + G)
+    counts = torch.randint(0, 5000, (G,), generator=g).to(dtype)
+    counts[torch.rand(G, generator=g) < 0.2] = 0
+    off = ops.group_offsets(counts.cuda()).cpu()
+    assert off.dtype == torch.int32 and off.numel() == G + 1
+    assert off.tolist() == [0] + np.cumsum(counts.numpy()).tolist()
+    with pytest.raises(RuntimeError, match="groups"):
+        ops.group_offsets(torch.zeros(257, dtype=torch.int32, device="cuda"))

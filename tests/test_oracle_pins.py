@@ -560,3 +560,150 @@ def test_gate_logits_spec_against_fp64_matmul():
     got_b = O.gate_logits_spec(x, wb, round_bf16=True)
     assert torch.equal(got_b, got_b.to(torch.bfloat16).float())
     assert float((got_b.double() - x.double() @ wb.double().t()).abs().max()) < 0.01 * float(ref.abs().max())
+
+
+def test_grouped_matmul_finalize_routing_closed_form():
+    """``grouped_matmul_finalize_routing`` (npu_grouped_matmul_finalize_routing, fused_moe.py:536) against an fp64
+    closed form that shares nothing with it: out[t] = shared[t - offset] + sum over the rows m with
+    row_index[m] == t of logit[m] * (a[m] . W[g(m)]) * w_scale[g(m)] * s[m], written with a Python loop over rows
+    and an exact integer product.  fp32 accumulation of at most K + 1 terms stays within a few ulp of it.
+    Must-fail variants: a wrong group's scale, the shared input at offset 0 instead of its offset, a missing logit.
+    For ``rows_bf16=True`` the rounding point is pinned: every row is rounded to bf16 *before* it is weighted;
+    rounding after the weighting gives other bits, and so does no rounding at all."""
+    g = torch.Generator().manual_seed(77)
+    G, Kd, H, T, off = 3, 64, 48, 12, 5
+    counts = torch.tensor([7, 0, 9])
+    M = int(counts.sum())
+    a = torch.randint(-128, 128, (M, Kd), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (G, Kd, H), generator=g, dtype=torch.int8)
+    w_scale = torch.rand(G, H, generator=g) * 1e-3 + 1e-4
+    s = torch.rand(M, generator=g) * 1e-2 + 1e-3
+    logit = torch.rand(M, generator=g) + 0.1
+    row_index = torch.randint(0, T, (M,), generator=g)
+    shared = (torch.randn(4, H, generator=g)).to(torch.bfloat16)      # rows [off, off + 4) of the output
+    got = O.grouped_matmul_finalize_routing(a, w, counts, w_scale, s, shared, logit, row_index, T, 1.0, off)
+    assert got.dtype == torch.float32 and tuple(got.shape) == (T, H)
+
+    def closed(scale_group_shift=0, shared_at=off, use_logit=True):
+        out = torch.zeros(T, H, dtype=torch.float64)
+        out[shared_at:shared_at + 4] += shared.double()
+        grp = torch.repeat_interleave(torch.arange(G), counts)
+        for m in range(M):
+            gm = int(grp[m])
+            acc = a[m].to(torch.int64) @ w[gm].to(torch.int64)            # exact
+            v = acc.double() * w_scale[(gm + scale_group_shift) % G].double() * float(s[m])
+            out[int(row_index[m])] += (float(logit[m]) if use_logit else 1.0) * v
+        return out
+    want = closed()
+    tol = 8 * torch.finfo(torch.float32).eps * want.abs().clamp(min=1e-30) + 1e-12
+    assert bool(((got.double() - want).abs() <= tol + 4e-7 * want.abs().max()).all())
+    rel = lambda x: float((got.double() - x).norm() / x.norm())
+    assert rel(want) < 1e-6
+    assert rel(closed(scale_group_shift=1)) > 1e-2          # a row dequantised with another group's scale
+    assert rel(closed(shared_at=0)) > 1e-2                  # the shared rows at offset 0 instead of `off`
+    assert rel(closed(use_logit=False)) > 1e-2              # the routing weight dropped
+    # rows outside [off, off + 4) start from zero, rows inside from the shared input: exact on a row nobody routes to
+    free = [t for t in range(T) if not bool((row_index == t).any())]
+    for t in free:
+        exp = shared[t - off].float() if off <= t < off + 4 else torch.zeros(H)
+        assert torch.equal(got[t], exp)
+
+    # ---- rows_bf16: rounding before the weight
+    got_bf = O.grouped_matmul_finalize_routing(a, w, counts, w_scale, s, shared, logit, row_index, T, 1.0, off,
+                                               rows_bf16=True)
+    acc = O.grouped_matmul_int32(a, w, counts)
+    grp = torch.repeat_interleave(torch.arange(G), counts)
+    deq = (acc.float() * w_scale[grp]) * s.unsqueeze(-1)                 # the operator's dequantisation (C8)
+
+    def combine(rows_fp32):
+        out = torch.zeros(T, H)
+        out[off:off + 4] = shared.float()
+        for m in range(M):                                               # ascending m, fp32, as the oracle states
+            out[int(row_index[m])] += rows_fp32[m]
+        return out
+    before = combine(logit.unsqueeze(-1) * deq.to(torch.bfloat16).float())
+    after = combine((logit.unsqueeze(-1) * deq).to(torch.bfloat16).float())
+    assert torch.equal(got_bf, before)
+    assert not torch.equal(got_bf, after) and not torch.equal(got_bf, got)
+    # and each rounded row is within half a bf16 step of the fp32 row it came from
+    assert bool(((deq.to(torch.bfloat16).float() - deq).abs() <= deq.abs() * 2.0 ** -8).all())
+
+
+def _a2_bruteforce(xq, xs, w1, w2, s1, s2, topk_w, topk_ids, expert_range, smooth, where="before"):
+    """fp64, permutation free, one expert at a time on the whole batch.  `where` places the smoothing factors:
+    "before" the row quantisation (the operator's order: quant_scale of npu_dequant_swiglu_quant), "none", or
+    "after" (on the quantised values instead) -- the last two are the mistakes the pin has to tell apart."""
+    lo, hi = expert_range
+    out = torch.zeros(xq.shape[0], w2.shape[2], dtype=torch.float64)
+    for e in range(lo, hi):
+        sel = topk_ids == e
+        tok = sel.any(dim=1)
+        if not bool(tok.any()):
+            continue
+        wt = (topk_w.double() * sel).sum(dim=1)[tok]
+        acc = xq[tok].to(torch.int64) @ w1[e - lo].to(torch.int64)
+        d = acc.double() * s1[e - lo].double() * xs[tok].double().unsqueeze(-1)
+        inter = d.shape[1] // 2
+        y = d[:, :inter] / (1.0 + torch.exp(-d[:, :inter])) * d[:, inter:]
+        if where == "before":
+            y = y * smooth[e - lo].double()
+        sc = y.abs().amax(dim=1) / 127.0
+        q = torch.round(y / sc.clamp(min=1e-300).unsqueeze(-1)).clamp(-128, 127)
+        if where == "after":
+            q = q * smooth[e - lo].double()
+        out[tok] += wt.unsqueeze(-1) * ((q @ w2[e - lo].double()) * s2[e - lo].double() * sc.unsqueeze(-1))
+    return out
+
+
+def test_a2_pipeline_against_bruteforce():
+    """``fused_experts_w8a8_allgather_ep_a2`` (fused_moe.py:844-937): with smoothing factors of one it is the A3
+    pipeline bit for bit (the reference's ``smooth_scale`` is ``torch.ones``, compressed_tensors_moe.py:113);
+    with other factors it follows the brute force that smooths before the row quantisation and not the ones that
+    drop the factors or apply them to the quantised values; the ``pd_seperate_prefill`` tail (bf16 rows, bf16
+    routing weights, bf16 w2 scale) stays within the bf16 bar of the same brute force and differs from the fp32
+    tail; an assignment outside the rank's range contributes nothing in either tail."""
+    T, K, n_local, E, H, I = 48, 4, 4, 16, 256, 128
+    lay = Layer(n_local, H, I, seed=31)
+    g = gen(32)
+    x = tokens(T, H, 33)
+    xq, xs = O.dynamic_quant(x)
+    ids = torch.rand(T, E, generator=g).argsort(1)[:, :K].int()
+    w = torch.rand(T, K, generator=g)
+    rng = (4, 4 + n_local)
+    ones = torch.ones(n_local, I)
+    a3 = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, rng)
+    a2 = O.fused_experts_w8a8_allgather_ep_a2(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, rng, ones)
+    assert torch.equal(a2, a3)
+    smooth = torch.rand(n_local, I, generator=g) * 1.5 + 0.25
+    got = O.fused_experts_w8a8_allgather_ep_a2(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, rng, smooth).double()
+    brute = {k: _a2_bruteforce(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, rng, smooth, k)
+             for k in ("before", "none", "after")}
+    assert rel_err(got, brute["before"]) < 5e-3
+    assert rel_err(got, brute["none"]) > 5e-2
+    # smoothing the quantised values differs from the operator's order by the quantisation noise only: small, but
+    # several times what separates the oracle from the brute force that has the order right
+    assert rel_err(got, brute["after"]) > 1e-2 > 2 * rel_err(got, brute["before"])
+    # tokens without a local expert get exactly zero
+    none_local = ~((ids >= rng[0]) & (ids < rng[1])).any(dim=1)
+    assert bool(none_local.any()) and bool((got[none_local] == 0).all())
+    # the bf16 tail
+    pd = O.fused_experts_w8a8_allgather_ep_a2(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, rng, smooth,
+                                              pd_seperate_prefill=True)
+    assert pd.dtype == torch.bfloat16 and rel_err(pd.double(), brute["before"]) < 1e-2
+    assert not torch.equal(pd.float(), got.float()) and bool((pd[none_local] == 0).all())
+    # its rounding points: rows to bf16 with a bf16 w2 scale, weights to bf16, fp32 sum in ascending k
+    _, st = O.fused_experts_w8a8_allgather_ep_a2(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, rng, smooth,
+                                                 pd_seperate_prefill=True, return_stages=True)
+    counts, idx = st["counts"], st["idx"].long()
+    acc2 = O.grouped_matmul_int32(st["h_q"], lay.w2_t, counts)
+    grp = torch.repeat_interleave(torch.arange(n_local), counts)
+    rows = ((acc2.float() * lay.s2.to(torch.bfloat16).float()[grp]) * st["h_s"].unsqueeze(-1)).to(torch.bfloat16)
+    slot_of = {int(s): m for m, s in enumerate(idx)}
+    want = torch.zeros(T, H)
+    wb = w.to(torch.bfloat16).float()
+    for n in range(T):
+        for k in range(K):
+            m = slot_of.get(n * K + k)
+            if m is not None:
+                want[n] += wb[n, k] * rows[m].float()
+    assert torch.equal(pd, want.to(torch.bfloat16))

@@ -42,6 +42,28 @@ def test_static_scratch_entry_matches_workspace_entry(rows_dtype):
         assert torch.equal(got, want), f"T={T}: static-scratch result differs from the workspace entry's"
 
 
+@pytest.mark.parametrize("case", ["int8_tokens", "no_shared_expert"])
+def test_static_scratch_entry_other_inputs(case):
+    """Tokens that arrive quantised (int8 + scales) and a layer without the shared expert (another scratch layout)
+    on the static scratch, two calls in a row, the second smaller: the bits of the workspace entry."""
+    from omni_infer_amd import hip_ops as ops
+    H, I, n, E, K = 2048, 1024, 8, 16, 4
+    with_shared = case != "no_shared_expert"
+    lay = Layer(n, H, I, seed=95, shared=with_shared)
+    d = lay.to_device()
+    shared = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"]) if with_shared else None
+    for T, seed in ((64, 96), (20, 97)):
+        x, w, ids = _inputs(T, H, E, K, n, seed)
+        xs = None
+        if case == "int8_tokens":
+            x, xs = ops.npu_dynamic_quant(x)
+        want = ops.moe_w8a8_layer(x, xs, w, ids, 0, n, d["w13"], d["s13"], d["w2"], d["s2"], shared, H=H, I=I)
+        out = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device="cuda")
+        got = ops.moe_w8a8_layer_static(x, xs, w, ids, 0, n, d["w13"], d["s13"], d["w2"], d["s2"], shared, H=H, I=I, out=out)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"{case} T={T}"
+
+
 def test_static_scratch_entry_rejects_what_does_not_fit():
     from omni_infer_amd import _lib as L
     from omni_infer_amd import hip_ops as ops
