@@ -149,15 +149,23 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
   for (int j = 0; j < NBF; ++j) wsv[j] = wsc[strip[j] * 16 + (lane & 15)];
 
-  // A rows this lane fetches when it stages fragments: row l%16 of each 16-row tile, k-step w of
-  // every chunk; rows past the end of the group alias the group's first row
+  // A staging.  A chunk of a 16-row tile is 16 rows x 256 bytes (4 k-steps); each wavefront fetches a quarter of
+  // it, one 16-byte piece per lane, and stores it where the MFMA operand reads expect it: k-step kk, lane slot
+  // 16 q + r for row r and k-quarter q.  GEMM1 (long rows, every block of a group re-reads the group's token rows
+  // from the L2): a wavefront takes 4 whole rows, i.e. 8 whole cache lines per load instruction (measured
+  // 1.8 us of the decode launch against the other split).  GEMM2: a wavefront takes one k-step of all 16 rows,
+  // 16 half lines, and its LDS stores are conflict free (measured 0.5 us better there).
+  // Rows past the end of the group alias the group's first row.
+  constexpr bool WHOLE_ROWS = (KIND == 1);
   const int8_t* arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    int rr = mt * 16 + (lane & 15);
+    int rr = mt * 16 + (WHOLE_ROWS ? 4 * w + (lane >> 4) : (lane & 15));
     if (rr >= nrows) rr = 0;
-    arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k64_0 * 64 + (lane >> 4) * 16 + w * 64;
+    arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k64_0 * 64 +
+               (WHOLE_ROWS ? (lane & 15) * 16 : (lane >> 4) * 16 + w * 64);
   }
+  const int a_slot = WHOLE_ROWS ? ((lane & 15) >> 2) * WAVE + (lane & 3) * 16 + 4 * w + (lane >> 4) : w * WAVE + lane;
 
   v4i acc[MT][NBF];
 #pragma unroll
@@ -170,7 +178,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt]);
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) lds_a[0][(mt * 4 + w) * WAVE + lane] = areg[mt];
+  for (int mt = 0; mt < MT; ++mt) lds_a[0][mt * 4 * WAVE + a_slot] = areg[mt];
   __syncthreads();
 
   // one chunk = 4 k-steps on ring slots [4*cc, 4*cc+4)
@@ -201,7 +209,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
     }
     v4i* ln = lds_a[(c + 1) & 1];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) ln[(mt * 4 + w) * WAVE + lane] = areg[mt];
+    for (int mt = 0; mt < MT; ++mt) ln[mt * 4 * WAVE + a_slot] = areg[mt];
     __syncthreads();
   };
 
