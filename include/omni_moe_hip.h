@@ -66,6 +66,9 @@ extern "C" {
                                      stays in the workspace, h_q / h_scale are not written.  The call is then
                                      exactly one kernel launch, which is how the benchmark times that kernel
                                      alone. */
+#define OMNI_GEMM1_WS_ZEROED 8    /* the caller has filled the workspace with zeros once and nothing but calls of this
+                                     entry with this flag and the same sizes have written to it since: the entry then
+                                     skips the launch that clears its arrival counters (it leaves them at zero) */
 /* combine: how src_to_dst is indexed */
 #define OMNI_IDX_TOKEN_MAJOR 0 /* n*K + k  (npu_moe_init_routing_v2 row_idx_type=1; finalize drop_pad_mode=2) */
 #define OMNI_IDX_K_MAJOR 1     /* k*T + n  (npu_moe_init_routing; finalize drop_pad_mode=0) */

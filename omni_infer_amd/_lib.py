@@ -54,7 +54,7 @@ SIGNATURES = {
 OMNI_DT_BF16, OMNI_DT_F32, OMNI_DT_F16 = 0, 1, 2
 OMNI_SCORE_SOFTMAX, OMNI_SCORE_SIGMOID = 0, 1
 OMNI_GROUP_MAX, OMNI_GROUP_TOP2SUM = 0, 1
-OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_REQUANT = 1, 4
+OMNI_GEMM1_BF16_INTERMEDIATE, OMNI_GEMM1_NO_REQUANT, OMNI_GEMM1_WS_ZEROED = 1, 4, 8
 OMNI_IDX_TOKEN_MAJOR, OMNI_IDX_K_MAJOR = 0, 1
 OMNI_ORDER_SLOT, OMNI_ORDER_K = 0, 1
 

@@ -263,13 +263,23 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
   int cnt_words = 0;
   size_t tail_bytes = 0;
   void* const tail = omni_tile_tail_area(T, K, G, extra, L.M_cap, H, I, ws + L.g1_ws, L.g1_bytes, &cnt_words, &tail_bytes);
+  // When GEMM1 runs the streaming kernel, the same kernel clears the arrival counters of its overflow blocks instead.
+  const omni_host::Plan p1 = omni_host::make_plan(1, T, K, G, extra, H, 2 * I);
+  const size_t bal_at = omni_host::gemm1_stream_bal_at(p1, L.M_cap, I);
+  int32_t* zero_words = (int32_t*)tail;
+  int zero_n = cnt_words;
+  if (!tail && bal_at != 0) {
+    zero_words = (int32_t*)(ws + L.g1_ws + bal_at);
+    zero_n = 2 * omni_host::STREAM_BAL_CNT_WORDS;
+  }
+  const bool counters_clean = zero_words != nullptr;
   bool routed = route == nullptr;
   if (route != nullptr && (x_dtype == OMNI_DT_BF16 || x_dtype == -1)) {
     // routing, quantisation (of bf16 tokens) and sort in one launch when the call is small
     const bool quantise = x_dtype == OMNI_DT_BF16;
     rc = omni_route_quant_permute_fused(route, quantise ? x : nullptr, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), K,
-                                        lo, hi, sorted_src, src_to_dst, (int32_t*)(ws + L.counts), offsets, (int32_t*)tail,
-                                        cnt_words, stream);
+                                        lo, hi, sorted_src, src_to_dst, (int32_t*)(ws + L.counts), offsets, zero_words,
+                                        zero_n, stream);
     if (rc < 0) return rc;
     routed = sorted = rc == 0;
     if (sorted && quantise) {
@@ -287,7 +297,7 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
     if (x_dtype == OMNI_DT_BF16)
       rc = omni_quant_permute_fused(x, T, H, (int8_t*)(ws + L.x_q), (float*)(ws + L.x_s), topk_ids, K, lo, hi,
                                     OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst, (int32_t*)(ws + L.counts), offsets,
-                                    (int32_t*)tail, cnt_words, stream);
+                                    zero_words, zero_n, stream);
     if (rc < 0) return rc;
     sorted = rc == 0;
     if (!sorted) {
@@ -299,13 +309,13 @@ int layer_impl(const void* x, int x_dtype, const float* x_scale_in, const float*
   }
   if (!sorted) {
     rc = omni_moe_permute_clearing(topk_ids, T, K, lo, hi, OMNI_IDX_TOKEN_MAJOR, sorted_src, src_to_dst,
-                                   (int32_t*)(ws + L.counts), offsets, ws + L.perm_ws, L.perm_bytes, (int32_t*)tail,
-                                   cnt_words, stream);
+                                   (int32_t*)(ws + L.counts), offsets, ws + L.perm_ws, L.perm_bytes, zero_words,
+                                   zero_n, stream);
     if (rc) return rc;
   }
   rc = omni_gemm1_swiglu_quant_impl(xq, xs, sorted_src, OMNI_IDX_TOKEN_MAJOR, T, K, w13_packed, w13_scale, sh13_packed,
                                     sh13_scale, extra, offsets, G, H, I, L.M_cap, 0, quant_scale, (int8_t*)(ws + L.h_q),
-                                    (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, tail != nullptr, stream);
+                                    (float*)(ws + L.h_s), nullptr, ws + L.g1_ws, L.g1_bytes, counters_clean, stream);
   if (rc) return rc;
   // The weighted sum rounds the shared expert's row to bf16 before it adds it to the rounded sum of the routed rows,
   // so with fp32 rows GEMM2 writes that group's rows as bf16 straight away (into the first half of the space their

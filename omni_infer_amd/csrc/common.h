@@ -69,6 +69,8 @@ int omni_moe_permute_clearing(const int32_t* topk_ids, int T, int K, int lo, int
 // library-internal (gemm.hip): the scratch of split tiles inside a GEMM1 workspace when both grouped GEMMs of a layer
 // call of this shape run the tile kernel (else null), with the number of counter words at its start that must be
 // zero before the first of the two launches; and the two GEMM entries with the promise that they are.
+// The same promise covers the counter words of the weight-streaming kernel's overflow blocks
+// (omni_host::gemm1_stream_bal_at: where they sit in a GEMM1 workspace).
 void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, void* gemm1_ws,
                           size_t gemm1_ws_bytes, int* counter_words, size_t* tail_bytes);
 int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const int32_t* sorted_src, int idx_mode, int T,

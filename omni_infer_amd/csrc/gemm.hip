@@ -1042,23 +1042,6 @@ Plan make_plan(int T, int K, int G, int extra_rows, int Kdim, int N, int64_t M_c
   return omni_host::make_plan(KIND, T, K, G, extra_rows, Kdim, N);
 }
 
-template <int KIND, int MT, int NT, int D>
-void launch_stream(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
-  GemmArgs a = a0;
-  const int BM = 16 * MT;
-  const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
-  int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
-  // GEMM1 (every block resident at once, long streams) gains from equal progress; GEMM2 (three rounds of short
-  // blocks, where the older round should finish first and make room) loses by it: measured 84.4 -> 87.6 us
-  a.equal_progress = (KIND == 1 && a.S == 1) ? (tuning().equal_progress & 1) : (tuning().equal_progress >> 1);
-  dim3 grid((unsigned)(units / (4 * NT)), (unsigned)mblocks, (unsigned)a.S), block(256);
-  hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
-}
-
-__global__ void zero_words_kernel(int32_t* p, int n) {
-  for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0;
-}
-
 // compute units of the current device (asked once per device)
 int device_cu_count() {
   static int cached[64];
@@ -1070,6 +1053,48 @@ int device_cu_count() {
     cached[dev] = n > 0 ? n : -1;
   }
   return cached[dev] > 0 ? cached[dev] : 0;
+}
+
+template <int KIND, int MT, int NT, int D>
+void launch_stream(const GemmArgs& a0, int64_t M_cap, int units, hipStream_t st) {
+  GemmArgs a = a0;
+  const int BM = 16 * MT;
+  const int Gt = a.G + (a.extra_rows > 0 ? 1 : 0);
+  int64_t mblocks = (M_cap + BM - 1) / BM + Gt;
+  // GEMM1 (every block resident at once, long streams) gains from equal progress; GEMM2 (three rounds of short
+  // blocks, where the older round should finish first and make room) loses by it: measured 84.4 -> 87.6 us
+  a.equal_progress = (KIND == 1 && a.S == 1) ? (tuning().equal_progress & 1) : (tuning().equal_progress >> 1);
+  const int cb = units / (4 * NT);
+  a.bal_cus = 0;
+  if (a.bal_cnt != nullptr && a.bal_part != nullptr && a.S == 1 && (KIND == 2 || a.y != nullptr) && tuning().stream_balance) {
+    // balanced numbering: needs the blocks a compute unit holds at once (asked once per variant)
+    static int resident = 0;
+    if (resident == 0) {
+      int n = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemm_stream<KIND, MT, NT, D>, 256, 0) != hipSuccess || n <= 0) n = -1;
+      resident = n;
+    }
+    const int cus = device_cu_count();
+    if (resident > 0 && cus > 0) {
+      constexpr size_t SHARE_BYTES = (size_t)4 * MT * ((KIND == 1) ? 2 * NT : NT) * 4 * WAVE * sizeof(int32_t);
+      const size_t cap = a.bal_part_bytes / SHARE_BYTES;
+      a.bal_cus = cus;
+      a.bal_resident = resident;
+      a.bal_cb = cb;
+      a.bal_share_cap = cap > 4096 ? 4096 : (int)cap;
+    }
+  }
+  if (a.bal_cus > 0) {
+    const int64_t nblocks = (int64_t)cb * mblocks + omni_host::stream_balance_max_helpers(a.bal_cus);
+    hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), dim3((unsigned)nblocks), dim3(256), 0, st, a);
+    return;
+  }
+  dim3 grid((unsigned)cb, (unsigned)mblocks, (unsigned)a.S), block(256);
+  hipLaunchKernelGGL((gemm_stream<KIND, MT, NT, D>), grid, block, 0, st, a);
+}
+
+__global__ void zero_words_kernel(int32_t* p, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0;
 }
 
 template <int KIND>
@@ -1177,9 +1202,13 @@ extern "C" int omni_moe_gemm1_swiglu_quant(const int8_t* x_q, const float* x_sca
                                            int H, int I, int64_t M_cap, int flags, const float* quant_scale,
                                            int8_t* h_q, float* h_scale, int32_t* acc_dbg, void* workspace,
                                            size_t ws_bytes, void* stream) {
+  // the promise of OMNI_GEMM1_WS_ZEROED is about the counters of the streaming kernel, which leaves them at zero; the
+  // tile kernel's are cleared in front of every launch
+  const bool zeroed = (flags & OMNI_GEMM1_WS_ZEROED) && T > 0 && K > 0 && G >= 0 && H > 0 && I > 0 &&
+                      !make_plan<1>(T, K, G, extra_rows, H, 2 * I, M_cap).tile;
   return omni_gemm1_swiglu_quant_impl(x_q, x_scale, sorted_src, idx_mode, T, K, w13_packed, w13_scale, w13_extra,
                                       w13_extra_scale, extra_rows, offsets, G, H, I, M_cap, flags, quant_scale, h_q,
-                                      h_scale, acc_dbg, workspace, ws_bytes, false, stream);
+                                      h_scale, acc_dbg, workspace, ws_bytes, zeroed, stream);
 }
 
 void* omni_tile_tail_area(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I, void* gemm1_ws,
@@ -1235,6 +1264,15 @@ int omni_gemm1_swiglu_quant_impl(const int8_t* x_q, const float* x_scale, const 
     // one k share: the stream kernel finishes y = silu(gate)*up itself (the workspace holds it, half
     // the bytes of the raw sums), then the row quantiser of the tile path
     a.y = (float*)workspace;
+    // overflow blocks of a launch that is resident at once are split along k: their counters and the scratch for
+    // the shares' partial sums end the workspace
+    const size_t bal_at = omni_host::gemm1_stream_bal_at(p, M_cap, I);
+    if (bal_at != 0 && tuning().stream_balance) {
+      a.bal_cnt = (int32_t*)((char*)workspace + bal_at);
+      a.bal_part = (int32_t*)((char*)workspace + bal_at + omni_host::STREAM_BAL_CNT_BYTES);
+      a.bal_part_bytes = omni_host::STREAM_BAL_PART_BYTES;
+      if (!counters_clean) hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(256), 0, st, a.bal_cnt, omni_host::STREAM_BAL_CNT_WORDS);
+    }
     rc = dispatch_gemm<1>(a, p, M_cap, nullptr, 0, false, st, "gemm1");
     if (rc) return rc;
     if (flags & OMNI_GEMM1_NO_REQUANT) return OMNI_OK;

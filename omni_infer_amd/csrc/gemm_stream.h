@@ -39,6 +39,13 @@ struct GemmArgs {
   int32_t* part;       // GEMM1 stream kernel: [S, M_cap, N] partial accumulators (split-k)
   int S;               // number of k splits (grid.z)
   int equal_progress;  // stream kernel: a wavefront lowers its issue priority as it advances through k
+  // stream kernel, balanced numbering (omni_host::stream_balance): compute units (0: the plain 3-d grid), blocks a
+  // unit holds at once, column blocks, shares the partial-sum scratch holds, the overflow blocks' arrival
+  // counters (zero at launch) and the scratch
+  int bal_cus, bal_resident, bal_cb, bal_share_cap;
+  int32_t* bal_cnt;
+  int32_t* bal_part;
+  size_t bal_part_bytes;  // host side only: bal_share_cap follows from it and the variant's block size
   int64_t M_cap;
 };
 
@@ -93,9 +100,53 @@ constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1
 // requested and before anything of A is touched: a caller whose A is still being produced waits there,
 // with its weight loads already in flight.  All four wavefronts of the block must call this together
 // (block barriers inside); when it returns nobody reads the LDS buffers any more.
+// Hand-over between the k shares of an overflow block (their blocks run on different compute units, possibly under
+// different L2s).  The partial sums are stored and loaded with device-scope accesses, word by word (written
+// through to where every L2 sees them, read past the caches), so that no bulk write-back or invalidation of
+// an L2 is needed in the middle of a launch that streams through it: every wavefront stores its sums and waits until
+// the stores are acknowledged, all wavefronts meet, one thread counts in at the block's counter.  True for the
+// share that arrived last: its accumulators then hold the sums of all shares.  Nobody waits for anybody.
+template <int MT, int NBF>
+__device__ __forceinline__ bool stream_handover(const GemmArgs& a, v4i (&acc)[MT][NBF], int over, int split, int share,
+                                                int w, int lane, int* s_last) {
+  constexpr int WAVE_INTS = MT * NBF * 4 * WAVE;
+  constexpr int BLOCK_INTS = 4 * WAVE_INTS;
+  int32_t* mine = a.bal_part + ((size_t)over * split + share) * BLOCK_INTS + (size_t)w * WAVE_INTS + lane;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int j = 0; j < NBF; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        __hip_atomic_store(mine + ((mt * NBF + j) * 4 + i) * WAVE, acc[mt][j][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0);  // every store of this wavefront has been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const bool last = __hip_atomic_fetch_add(a.bal_cnt + over, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == split - 1;
+    // nobody else touches the word any more in this launch: it is left at zero for the next one
+    if (last) __hip_atomic_store(a.bal_cnt + over, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_last = last;
+  }
+  __syncthreads();
+  if (!*s_last) return false;
+  for (int s2 = 0; s2 < split; ++s2) {
+    if (s2 == share) continue;
+    const int32_t* theirs = a.bal_part + ((size_t)over * split + s2) * BLOCK_INTS + (size_t)w * WAVE_INTS + lane;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < NBF; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[mt][j][i] += __hip_atomic_load(theirs + ((mt * NBF + j) * 4 + i) * WAVE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  return true;
+}
+
+// k share `bz` of `nz`; over >= 0: the block is one share of overflow block `over` and hands its sums over
 template <int KIND, int MT, int NT, int D, typename BeforeA>
-__device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& rb, int bx, int bz,
-                                             v4i (*lds_a)[MT * 4 * WAVE], float* lds_ts, BeforeA before_a) {
+__device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& rb, int bx, int bz, int nz, int over,
+                                             int* s_last, v4i (*lds_a)[MT * 4 * WAVE], float* lds_ts, BeforeA before_a) {
   constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
   constexpr int DC = D / 4;                       // chunks (4 k-steps) of B in flight
   static_assert(D % 4 == 0, "D counts whole chunks");
@@ -105,7 +156,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int mt_cnt = (nrows + 15) / 16;
   const int nk64_all = a.Kdim / 64;          // k-steps of the whole reduction
-  const int nk64 = nk64_all / a.S;           // k-steps of this block's share
+  const int nk64 = nk64_all / nz;            // k-steps of this block's share
   const int k64_0 = bz * nk64;
   const int nchunks = nk64 / 4;
   const int I = (KIND == 1) ? a.N / 2 : 0;
@@ -234,6 +285,9 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
   for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, false);
 
+  if (over >= 0) {
+    if (!stream_handover<MT, NBF>(a, acc, over, nz, bz, w, lane, s_last)) return;
+  }
   // ---- epilogue
   const int col = lane & 15;
   if constexpr (KIND == 1) {
@@ -308,9 +362,23 @@ template <int KIND, int MT, int NT, int D>
 __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void gemm_stream(GemmArgs a) {
   __shared__ v4i lds_a[2][MT * 4 * WAVE];
   __shared__ float lds_ts[16 * MT];
+  __shared__ int s_last;
   RowBlock rb;
+  if (a.bal_cus > 0) {
+    // 1-d grid, balanced numbering: whole blocks, the overflow blocks' first shares, the helper shares
+    const RowBlockScan sc = row_blocks_scan(a.offsets, a.G, a.extra_rows, 16 * MT);
+    const int n_real = sc.total * a.bal_cb;
+    const omni_host::StreamBalance bal =
+        omni_host::stream_balance(n_real, a.bal_cus, a.bal_resident, a.Kdim / 256, D / 4, a.bal_share_cap);
+    omni_host::StreamSel sel;
+    if (!omni_host::stream_select(bal, n_real, (int)blockIdx.x, sel)) return;
+    if (!row_blocks_find(sc, a.offsets, a.G, a.extra_rows, 16 * MT, sel.task / a.bal_cb, rb)) return;
+    stream_block<KIND, MT, NT, D>(a, rb, sel.task % a.bal_cb, sel.share, sel.over >= 0 ? bal.split : 1, sel.over, &s_last,
+                                  lds_a, lds_ts, [] {});
+    return;
+  }
   if (!find_row_block(a.offsets, a.G, a.extra_rows, 16 * MT, blockIdx.y, rb)) return;
-  stream_block<KIND, MT, NT, D>(a, rb, blockIdx.x, blockIdx.z, lds_a, lds_ts, [] {});
+  stream_block<KIND, MT, NT, D>(a, rb, blockIdx.x, blockIdx.z, a.S, -1, &s_last, lds_a, lds_ts, [] {});
 }
 
 // Row quantisation of y = silu(gate) * up (fp32) by one wavefront: scale = max|y| / 127, q = rint(y / scale).

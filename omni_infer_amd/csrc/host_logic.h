@@ -143,6 +143,59 @@ OMNI_HD void tile_share_k_range(int nk, int ku, int split, int share, int& k_fir
 }
 
 // ------------------------------------------------------------------------------------------------
+// Block numbering of the weight-streaming kernel when the whole launch is resident at once
+// A compute unit draws at most about 30 GB/s from memory, a ninth above its share of what the chip delivers
+// when every unit pulls (27 GB/s of 6.97 TB/s); blocks stay where the dispatcher puts them.  A launch of
+// q * cus + r blocks therefore leaves r units with q + 1 blocks and runs as long as those take: 33 x 32 blocks of
+// the decode GEMM1 read at 6.45 TB/s where 32 x 32 read at 6.95 (measured with a kernel that only reads).
+// So the last r blocks ("overflow") are each cut `split` ways along the reduction: the block itself takes the
+// first share, helper blocks with the ids [n_real, n_real + r * (split - 1)) the others, every unit ends up
+// with q blocks and a few shares, and whoever arrives last at an overflow block's counter adds up the partial
+// sums (integers: any order) and runs the epilogue.
+// ------------------------------------------------------------------------------------------------
+// arrival counters of the overflow blocks: one word each, GEMM1's and GEMM2's apart (one clearing serves both)
+constexpr int STREAM_BAL_CNT_WORDS = 256;   // per kind of GEMM; a launch with more overflow blocks is not split
+struct StreamBalance { int cap, n_over, split, total; };  // ids [0, cap) whole blocks; n_over overflow blocks; all ids
+struct StreamSel { int task, share, over; };              // block of the launch, its k share, overflow index or -1
+
+// n_real: blocks with rows; resident: blocks a unit holds at once; nchunks: chunks of 4 k-steps of the reduction;
+// dc: chunks a wavefront keeps in flight; share_cap: shares the partial-sum scratch holds (0: no scratch)
+OMNI_HD StreamBalance stream_balance(int n_real, int cus, int resident, int nchunks, int dc, int share_cap) {
+  StreamBalance b{n_real, 0, 1, n_real};
+  if (cus <= 0 || n_real <= cus || share_cap <= 0) return b;
+  const int q = n_real / cus, r = n_real % cus;
+  if (r == 0 || q + 1 > resident) return b;           // even already, or more than one round: the dispatcher evens out
+  if (r > STREAM_BAL_CNT_WORDS) return b;
+  if (100 * (q + 1) * cus < 104 * n_real) return b;   // the fullest unit is within 4 % of the mean
+  int split = 0;
+  for (int sp = 4; sp >= 2; sp -= 2)
+    if (nchunks % sp == 0 && nchunks / sp >= 2 * dc && r * sp <= share_cap) { split = sp; break; }
+  if (split == 0) return b;
+  b.cap = n_real - r;
+  b.n_over = r;
+  b.split = split;
+  b.total = n_real + r * (split - 1);
+  return b;
+}
+OMNI_HD bool stream_select(const StreamBalance& b, int n_real, int id, StreamSel& s) {
+  s.task = id;
+  s.share = 0;
+  s.over = -1;
+  if (id < 0 || id >= b.total) return false;
+  if (id >= n_real) {
+    const int h = id - n_real;            // helper: consecutive ids serve different overflow blocks
+    s.over = h % b.n_over;
+    s.share = 1 + h / b.n_over;
+    s.task = b.cap + s.over;
+  } else if (id >= b.cap) {
+    s.over = id - b.cap;
+  }
+  return true;
+}
+// most helper blocks a launch can need
+OMNI_HD int stream_balance_max_helpers(int cus) { return cus > 1 ? (cus - 1) * 3 : 0; }
+
+// ------------------------------------------------------------------------------------------------
 // Kernel choice of the grouped GEMMs and what follows from it
 // ------------------------------------------------------------------------------------------------
 // Tuning aids, read from the environment once (the first GEMM call of the process) and never again:
@@ -155,11 +208,13 @@ OMNI_HD void tile_share_k_range(int nk, int ku, int split, int share, int& k_fir
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
+//   OMNI_MOE_STREAM_BALANCE 0: the overflow blocks of a resident stream launch are not split along k
 //   OMNI_MOE_EQUAL_PROGRESS bit 0: the stream kernel of GEMM1 lowers the issue priority of its wavefronts as they
 //                          advance (default 1), bit 1: that of GEMM2 too (measured slower in every geometry)
 struct Tuning {
   int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
   int tile_mfma16 = 1;
+  int stream_balance = 1;
   bool have[3] = {false, false, false};
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
@@ -191,6 +246,7 @@ inline Tuning read_tuning() {
   r.rowq = geti("OMNI_MOE_ROWQ", 0);
   r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
   r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
+  r.stream_balance = geti("OMNI_MOE_STREAM_BALANCE", 1);
   for (int kind = 1; kind <= 2; ++kind) {
     const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
     const char* e = getenv(name);
@@ -284,12 +340,25 @@ constexpr size_t TILE_TAIL_BYTES = TILE_TAIL_CNT_BYTES + TILE_TAIL_PART_BYTES;
 // the entry on the library's static scratch refuses every shape that selects the tile kernel by size alone
 static_assert(TILE_TAIL_BYTES > (size_t)OMNI_STATIC_SCRATCH_BYTES, "a tile-kernel call must not fit the static scratch");
 
+// Scratch of the overflow blocks of a stream launch (stream_balance): the counter words of GEMM1 and of GEMM2,
+// then room for the partial sums of the k shares.  It ends the GEMM1 workspace of a stream plan with one k share.
+constexpr size_t STREAM_BAL_PART_BYTES = (size_t)8 << 20;
+constexpr size_t STREAM_BAL_CNT_BYTES = 2 * STREAM_BAL_CNT_WORDS * sizeof(int32_t);
+constexpr size_t STREAM_BAL_BYTES = STREAM_BAL_CNT_BYTES + STREAM_BAL_PART_BYTES;
+inline size_t gemm1_stream_sums_bytes(const Plan& p, int64_t M_cap, int I) {
+  return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
+}
+// byte offset of that scratch in the GEMM1 workspace, or 0 when the plan has none
+inline size_t gemm1_stream_bal_at(const Plan& p, int64_t M_cap, int I) {
+  return (!p.tile && p.S == 1) ? align256(gemm1_stream_sums_bytes(p, M_cap, I)) : 0;
+}
 inline size_t gemm1_ws_bytes(const Plan& p, int64_t M_cap, int I) {
   if (p.tile) {
     // y = silu(gate) * up before the row quantiser, then the scratch of the split tiles
     return align256((size_t)M_cap * I * sizeof(float) + 256) + TILE_TAIL_BYTES;
   }
-  return (size_t)p.S * M_cap * 2 * I * sizeof(int32_t) + 256;
+  const size_t at = gemm1_stream_bal_at(p, M_cap, I);
+  return at ? at + STREAM_BAL_BYTES : gemm1_stream_sums_bytes(p, M_cap, I);
 }
 inline size_t gemm1_workspace_bytes(int T, int K, int G, int extra_rows, int64_t M_cap, int H, int I) {
   if (M_cap < 0 || I <= 0 || H <= 0 || T < 0 || K <= 0 || G < 0) return 0;

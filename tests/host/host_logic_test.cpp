@@ -266,6 +266,56 @@ static void test_tiles(std::mt19937& rng) {
       }
 }
 
+// Balanced numbering of the weight-streaming kernel: every block of the launch is covered by exactly the k-steps
+// of its reduction, once; helper ids stay inside the grid the host launches; the overflow blocks fit the counter
+// words and the partial-sum scratch; after the split no unit is more than a quarter block above the mean.
+static void test_stream_balance(std::mt19937& rng) {
+  for (int it = 0; it < 20000; ++it) {
+    const int cus = (it % 3 == 0) ? 256 : 1 + (int)(rng() % 320);
+    const int n_real = (it % 5 == 0) ? 1024 + (int)(rng() % 300) : (int)(rng() % 4000);
+    const int resident = 1 + (int)(rng() % 8), dc = 1 + (int)(rng() % 2);
+    const int nchunks = dc * (1 + (int)(rng() % 28));
+    const int share_cap = (rng() % 4 == 0) ? 0 : (int)(rng() % 2000);
+    const StreamBalance b = stream_balance(n_real, cus, resident, nchunks, dc, share_cap);
+    CHECK(b.split == 1 || b.split == 2 || b.split == 4);
+    CHECK(b.cap + b.n_over == n_real);
+    CHECK(b.total == n_real + b.n_over * (b.split - 1));
+    CHECK(b.total - n_real <= stream_balance_max_helpers(cus));
+    if (b.split > 1) {
+      CHECK(b.n_over > 0 && b.n_over < cus && b.n_over <= STREAM_BAL_CNT_WORDS);
+      CHECK(b.n_over * b.split <= share_cap);
+      CHECK(nchunks % b.split == 0 && nchunks / b.split >= 2 * dc);
+      CHECK(b.cap % cus == 0 && b.cap / cus + 1 <= resident);
+    } else {
+      CHECK(b.n_over == 0);
+    }
+    std::vector<int> covered(n_real, 0);   // k shares seen per block, as a bit mask
+    for (int id = -1; id < b.total + 3; ++id) {
+      StreamSel s;
+      const bool ok = stream_select(b, n_real, id, s);
+      CHECK(ok == (id >= 0 && id < b.total));
+      if (!ok) continue;
+      CHECK(s.task >= 0 && s.task < n_real);
+      if (s.task < b.cap) {
+        CHECK(s.over == -1 && s.share == 0);
+        covered[s.task] |= 0xf;
+      } else {
+        CHECK(s.over == s.task - b.cap && s.share >= 0 && s.share < b.split);
+        CHECK(!(covered[s.task] & (1 << s.share)));
+        covered[s.task] |= 1 << s.share;
+      }
+    }
+    for (int t = 0; t < n_real; ++t) CHECK(covered[t] == (t < b.cap ? 0xf : (1 << b.split) - 1));
+  }
+  // the decode shape: 34 row blocks x 32 column blocks on 256 units that hold 5 blocks each
+  const StreamBalance d = stream_balance(1088, 256, 5, 28, 1, 4096);
+  CHECK(d.cap == 1024 && d.n_over == 64 && d.split == 4 && d.total == 1088 + 192);
+  CHECK(stream_balance(1024, 256, 5, 28, 1, 4096).split == 1);    // even already
+  CHECK(stream_balance(1280 + 64, 256, 5, 28, 1, 4096).split == 1);   // a second round: left to the dispatcher
+  CHECK(stream_balance(1088, 256, 5, 28, 1, 100).split == 1);     // scratch too small for 64 x 2 shares
+  CHECK(stream_balance(1088, 256, 5, 28, 1, 200).split == 2);
+}
+
 static void test_layout(std::mt19937& rng) {
   for (int it = 0; it < 2000; ++it) {
     const int T = 1 + rng() % ((it % 10 == 0) ? 20000 : 600);
@@ -294,6 +344,12 @@ static void test_layout(std::mt19937& rng) {
     const Plan p1 = make_plan(1, T, K, G, with_shared ? T : 0, H, 2 * I);
     if (p1.tile) CHECK(L.g1_bytes >= (size_t)M_cap * I * 4 + TILE_TAIL_BYTES);
     else CHECK(L.g1_bytes >= (size_t)p1.S * M_cap * 2 * I * 4);
+    if (!p1.tile && p1.S == 1) {   // the scratch of the overflow blocks ends the workspace, past the sums, aligned
+      const size_t at = gemm1_stream_bal_at(p1, M_cap, I);
+      CHECK(at % 256 == 0 && at >= (size_t)M_cap * 2 * I * 4 && at + STREAM_BAL_BYTES <= L.g1_bytes);
+    } else {
+      CHECK(gemm1_stream_bal_at(p1, M_cap, I) == 0);
+    }
     if (!p1.tile) CHECK(stream_variant_exists(1, p1.mt, p1.nt, p1.d));
     const Plan p2 = make_plan(2, (int)M_cap, 1, G, with_shared ? T : 0, I, H);
     if (!p2.tile) CHECK(stream_variant_exists(2, p2.mt, p2.nt, p2.d));
@@ -377,6 +433,7 @@ int main() {
   std::mt19937 rng(12345);
   test_row_blocks(rng);
   test_tiles(rng);
+  test_stream_balance(rng);
   test_layout(rng);
   test_arrive_book();
   test_placement(rng);
