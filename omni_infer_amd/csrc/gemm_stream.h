@@ -70,7 +70,10 @@ __device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float ws
     if (rr < nrows) {
       float o = ((float)acc[i] * ws) * ts[i];
       size_t m = (size_t)(row0 + rr);
-      if (a.out_dtype == OMNI_DT_F32) ((float*)a.rows_out)[m * (size_t)a.N + n] = o;
+      // fp32 rows are written through (a device-scope store): the combine reads them under every L2, and the launch
+      // does not end on the write-back of 16 MB of dirty lines (measured: 1.3 us off the decode layer)
+      if (a.out_dtype == OMNI_DT_F32)
+        __hip_atomic_store((float*)a.rows_out + m * (size_t)a.N + n, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else ((uint16_t*)a.rows_out)[m * (size_t)a.N + n] = f32_to_bf16(o);
       if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + n] = acc[i];
     }
@@ -95,11 +98,6 @@ __device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float ws
 template <int KIND, int MT, int NT, int D>
 constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1; }
 
-// One block's work: the rows of row block `rb` times the channels of column block `bx` (4 wavefronts x NT
-// strips, or strip pairs), k share `bz` of a.S.  `before_a()` runs after the first D k-steps of B have been
-// requested and before anything of A is touched: a caller whose A is still being produced waits there,
-// with its weight loads already in flight.  All four wavefronts of the block must call this together
-// (block barriers inside); when it returns nobody reads the LDS buffers any more.
 // Hand-over between the k shares of an overflow block (their blocks run on different compute units, possibly under
 // different L2s).  The partial sums are stored and loaded with device-scope accesses, word by word (written
 // through to where every L2 sees them, read past the caches), so that no bulk write-back or invalidation of
@@ -143,7 +141,12 @@ __device__ __forceinline__ bool stream_handover(const GemmArgs& a, v4i (&acc)[MT
   return true;
 }
 
-// k share `bz` of `nz`; over >= 0: the block is one share of overflow block `over` and hands its sums over
+// One block's work: the rows of row block `rb` times the channels of column block `bx` (4 wavefronts x NT
+// strips, or strip pairs), k share `bz` of `nz`; over >= 0: the block is one share of overflow block `over` and
+// hands its sums over.  `before_a()` runs after the first D k-steps of B have been requested and before anything
+// of A is touched: a caller whose A is still being produced waits there, with its weight loads already in
+// flight.  All four wavefronts of the block must call this together (block barriers inside); when it returns
+// nobody reads the LDS buffers any more.
 template <int KIND, int MT, int NT, int D, typename BeforeA>
 __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& rb, int bx, int bz, int nz, int over,
                                              int* s_last, v4i (*lds_a)[MT * 4 * WAVE], float* lds_ts, BeforeA before_a) {
