@@ -372,7 +372,8 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
     const RowBlockScan sc = row_blocks_scan(a.offsets, a.G, a.extra_rows, 16 * MT);
     const int n_real = sc.total * a.bal_cb;
     const omni_host::StreamBalance bal =
-        omni_host::stream_balance(n_real, a.bal_cus, a.bal_resident, a.Kdim / 256, D / 4, a.bal_share_cap);
+        omni_host::stream_balance(n_real, a.bal_cus, a.bal_resident, a.Kdim / 256, D / 4, a.bal_share_cap,
+                                  ((KIND == 1) ? 2 * NT : NT) * a.Kdim / 16);
     omni_host::StreamSel sel;
     if (!omni_host::stream_select(bal, n_real, (int)blockIdx.x, sel)) return;
     if (!row_blocks_find(sc, a.offsets, a.G, a.extra_rows, 16 * MT, sel.task / a.bal_cb, rb)) return;

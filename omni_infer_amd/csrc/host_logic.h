@@ -158,18 +158,37 @@ constexpr int STREAM_BAL_CNT_WORDS = 256;   // per kind of GEMM; a launch with m
 struct StreamBalance { int cap, n_over, split, total; };  // ids [0, cap) whole blocks; n_over overflow blocks; all ids
 struct StreamSel { int task, share, over; };              // block of the launch, its k share, overflow index or -1
 
+// Whether the cut pays, and how many shares: in units of the time a busy compute unit takes for one block, the
+// launch takes q + 1 without the cut; with `sp` shares per overflow block it takes what the fullest unit then holds,
+// q + ceil(r sp / cus) / sp, but no less than 1.08 times the mean load q + r / cus (a unit alone draws about a
+// tenth more than its share of the chip's rate), plus what a share costs on top of its bytes (its first loads, the
+// hand-over of its partial sums: 2.7 us measured, which a busy unit streams 83 KB in) for every share a unit gets.
+// The cut is made when the best `sp` saves at least 2 % of a block's time.  The two constants were set on the
+// DeepSeek-V3 GEMM1 (917 KB blocks, 256 units) and give the sign of all sixteen measured cases: layer time with 2 /
+// 4 shares against uncut at 1 token (9 x 32 blocks) -7.0 / -10.0 us, 2 tokens (14 x 32) +6.6 / +5.2, 4 tokens (21 x 32)
+// +5.8 / +5.8, 8 tokens (31 x 32) +4.9 / +11.4, 16 tokens (33 x 32) -7.0 / -9.1, 32 tokens -5.5 / -5.6, 64 tokens
+// (34 x 32) -7.2 / -6.1, 96 tokens (36 x 32) -3.7 / +2.4.
 // n_real: blocks with rows; resident: blocks a unit holds at once; nchunks: chunks of 4 k-steps of the reduction;
-// dc: chunks a wavefront keeps in flight; share_cap: shares the partial-sum scratch holds (0: no scratch)
-OMNI_HD StreamBalance stream_balance(int n_real, int cus, int resident, int nchunks, int dc, int share_cap) {
+// dc: chunks a wavefront keeps in flight; share_cap: shares the partial-sum scratch holds (0: no scratch);
+// block_kb: weight bytes a block streams, in KiB
+OMNI_HD StreamBalance stream_balance(int n_real, int cus, int resident, int nchunks, int dc, int share_cap, int block_kb) {
   StreamBalance b{n_real, 0, 1, n_real};
-  if (cus <= 0 || n_real <= cus || share_cap <= 0) return b;
+  if (cus <= 0 || n_real <= cus || share_cap <= 0 || block_kb <= 0) return b;
   const int q = n_real / cus, r = n_real % cus;
   if (r == 0 || q + 1 > resident) return b;           // even already, or more than one round: the dispatcher evens out
   if (r > STREAM_BAL_CNT_WORDS) return b;
-  if (100 * (q + 1) * cus < 104 * n_real) return b;   // the fullest unit is within 4 % of the mean
+  // everything in thousandths of a block's time
+  const long long whole = 1000LL * (q + 1);
+  const long long mean_floor = 1080LL * n_real / cus;
+  long long best = whole - 20;
   int split = 0;
-  for (int sp = 4; sp >= 2; sp -= 2)
-    if (nchunks % sp == 0 && nchunks / sp >= 2 * dc && r * sp <= share_cap) { split = sp; break; }
+  for (int sp = 2; sp <= 4; sp += 2) {
+    if (nchunks % sp != 0 || nchunks / sp < 2 * dc || r * sp > share_cap) continue;
+    const long long shares_per_unit = ((long long)r * sp + cus - 1) / cus;
+    const long long fullest = 1000LL * q + 1000LL * shares_per_unit / sp;
+    const long long cost = (fullest > mean_floor ? fullest : mean_floor) + 83LL * 1000 * r * sp / ((long long)cus * block_kb);
+    if (cost < best) { best = cost; split = sp; }
+  }
   if (split == 0) return b;
   b.cap = n_real - r;
   b.n_over = r;

@@ -276,7 +276,8 @@ static void test_stream_balance(std::mt19937& rng) {
     const int resident = 1 + (int)(rng() % 8), dc = 1 + (int)(rng() % 2);
     const int nchunks = dc * (1 + (int)(rng() % 28));
     const int share_cap = (rng() % 4 == 0) ? 0 : (int)(rng() % 2000);
-    const StreamBalance b = stream_balance(n_real, cus, resident, nchunks, dc, share_cap);
+    const int block_kb = 1 + (int)(rng() % 2000);
+    const StreamBalance b = stream_balance(n_real, cus, resident, nchunks, dc, share_cap, block_kb);
     CHECK(b.split == 1 || b.split == 2 || b.split == 4);
     CHECK(b.cap + b.n_over == n_real);
     CHECK(b.total == n_real + b.n_over * (b.split - 1));
@@ -307,13 +308,21 @@ static void test_stream_balance(std::mt19937& rng) {
     }
     for (int t = 0; t < n_real; ++t) CHECK(covered[t] == (t < b.cap ? 0xf : (1 << b.split) - 1));
   }
-  // the decode shape: 34 row blocks x 32 column blocks on 256 units that hold 5 blocks each
-  const StreamBalance d = stream_balance(1088, 256, 5, 28, 1, 4096);
-  CHECK(d.cap == 1024 && d.n_over == 64 && d.split == 4 && d.total == 1088 + 192);
-  CHECK(stream_balance(1024, 256, 5, 28, 1, 4096).split == 1);    // even already
-  CHECK(stream_balance(1280 + 64, 256, 5, 28, 1, 4096).split == 1);   // a second round: left to the dispatcher
-  CHECK(stream_balance(1088, 256, 5, 28, 1, 100).split == 1);     // scratch too small for 64 x 2 shares
-  CHECK(stream_balance(1088, 256, 5, 28, 1, 200).split == 2);
+  // GEMM1 of the DeepSeek-V3 shape (blocks of 917 KB, 28 chunks) on 256 units that hold 5 blocks each
+  const StreamBalance d = stream_balance(1088, 256, 5, 28, 1, 1024, 896);   // 64 tokens: 34 row blocks x 32
+  CHECK(d.cap == 1024 && d.n_over == 64 && d.split == 2 && d.total == 1088 + 64);
+  CHECK(stream_balance(1056, 256, 5, 28, 1, 1024, 896).split == 4);   // 16 and 32 tokens
+  CHECK(stream_balance(288, 256, 7, 28, 1, 1024, 896).split == 4);    // 1 token
+  CHECK(stream_balance(448, 256, 7, 28, 1, 1024, 896).split == 1);    // 2, 4 and 8 tokens: the chip's rate is reached
+  CHECK(stream_balance(672, 256, 7, 28, 1, 1024, 896).split == 1);    //   uncut, or the shares cost more than they save
+  CHECK(stream_balance(992, 256, 7, 28, 1, 1024, 896).split == 1);
+  CHECK(stream_balance(1152, 256, 5, 28, 1, 1024, 896).split == 2);   // 96 tokens: halves pay, quarters do not
+  CHECK(stream_balance(1216, 256, 5, 28, 1, 1024, 896).split == 1);   // the fullest unit is near the mean
+  CHECK(stream_balance(1024, 256, 5, 28, 1, 1024, 896).split == 1);   // even already
+  CHECK(stream_balance(1280 + 64, 256, 5, 28, 1, 1024, 896).split == 1);   // a second round: left to the dispatcher
+  CHECK(stream_balance(1088, 256, 5, 28, 1, 100, 896).split == 1);    // scratch too small for 64 x 2 shares
+  CHECK(stream_balance(1056, 256, 5, 28, 1, 100, 896).split == 2);    // room for 32 x 2 shares, not for 32 x 4
+  CHECK(stream_balance(1088, 256, 5, 28, 1, 1024, 16).split == 1);    // tiny blocks: a share costs more than it saves
 }
 
 static void test_layout(std::mt19937& rng) {
