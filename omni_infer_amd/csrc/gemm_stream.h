@@ -2,6 +2,7 @@
 // GEMM kernels: the argument record, the source-row lookup and the GEMM2 row epilogue.
 #pragma once
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -62,22 +63,32 @@ __device__ __forceinline__ int source_row(const GemmArgs& a, int g, int r) {
   }
 }
 
+// GEMM2 rows of one accumulator tile of a lane: rows rbase .. rbase + 3 of the block, channel n.  The output type is
+// a template parameter and the address of a row follows from the one above it, so that a row costs one add, one
+// compare and one store.
+// fp32 rows are written through (a device-scope store): the combine reads them under every L2, and the launch
+// does not end on the write-back of 16 MB of dirty lines (measured: 1.3 us off the decode layer).
+template <bool F32>
 __device__ __forceinline__ void epilogue_gemm2(const GemmArgs& a, const float ws, int n, int row0, int rbase,
                                                int nrows, const float* ts, v4i acc) {
+  using Out = typename std::conditional<F32, float, uint16_t>::type;
+  Out* p = (Out*)a.rows_out + (size_t)(row0 + rbase) * (size_t)a.N + n;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    int rr = rbase + i;
-    if (rr < nrows) {
-      float o = ((float)acc[i] * ws) * ts[i];
-      size_t m = (size_t)(row0 + rr);
-      // fp32 rows are written through (a device-scope store): the combine reads them under every L2, and the launch
-      // does not end on the write-back of 16 MB of dirty lines (measured: 1.3 us off the decode layer)
-      if (a.out_dtype == OMNI_DT_F32)
-        __hip_atomic_store((float*)a.rows_out + m * (size_t)a.N + n, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      else ((uint16_t*)a.rows_out)[m * (size_t)a.N + n] = f32_to_bf16(o);
-      if (a.acc_dbg) a.acc_dbg[m * (size_t)a.N + n] = acc[i];
+    if (rbase + i < nrows) {
+      const float o = ((float)acc[i] * ws) * ts[i];
+      if constexpr (F32) __hip_atomic_store(p, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else *p = f32_to_bf16(o);
     }
+    p += a.N;
   }
+}
+// raw accumulators for the parity tests, kept out of the epilogue so that none of their address arithmetic is
+// ever part of it
+__device__ __forceinline__ void dump_acc_gemm2(const GemmArgs& a, int n, int row0, int rbase, int nrows, v4i acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (rbase + i < nrows) a.acc_dbg[(size_t)(row0 + rbase + i) * (size_t)a.N + n] = acc[i];
 }
 
 // =====================================================================================
@@ -347,6 +358,7 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
       }
     }
   } else {
+    const bool f32_rows = a.out_dtype == OMNI_DT_F32;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       if (mt < mt_cnt) {
@@ -355,7 +367,11 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
         for (int i = 0; i < 4; ++i) ts[i] = lds_ts[rbase + i];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) epilogue_gemm2(a, wsv[t], strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
+        for (int t = 0; t < NT; ++t) {
+          if (f32_rows) epilogue_gemm2<true>(a, wsv[t], strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
+          else epilogue_gemm2<false>(a, wsv[t], strip[t] * 16 + col, row0, rbase, nrows, ts, acc[mt][t]);
+          if (a.acc_dbg) dump_acc_gemm2(a, strip[t] * 16 + col, row0, rbase, nrows, acc[mt][t]);
+        }
       }
     }
   }
