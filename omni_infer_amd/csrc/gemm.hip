@@ -1156,6 +1156,10 @@ int dispatch_gemm(const GemmArgs& a, const Plan& p, int64_t M_cap, void* tail_ws
     const int mt = p.mt, nt = p.nt, d = p.d;
     if (units % (4 * nt) != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: %d output strips not divisible by %d", what, units, 4 * nt);
     if (a.Kdim % 256 != 0) OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: reduction length %d must be a multiple of 256", what, a.Kdim);
+    // the stream kernel addresses its activation operand with 32-bit byte offsets
+    const int64_t a_rows = (KIND == 1) ? (int64_t)a.T : M_cap;
+    if (a_rows * a.Kdim >= ((int64_t)1 << 32))
+      OMNI_FAIL(OMNI_E_UNSUPPORTED, "%s: %lld rows of %d bytes are too many for the small-batch kernel", what, (long long)a_rows, a.Kdim);
     bool ok = false;
 #define TRY(K_, MT_, NT_, D_)                                                  \
   if (!ok && KIND == K_ && mt == MT_ && nt == NT_ && d == D_) {                \

@@ -107,7 +107,12 @@ __device__ __forceinline__ void dump_acc_gemm2(const GemmArgs& a, int n, int row
 // registers) so that a decode-sized launch (about 34 row blocks x 32 channel blocks) is resident
 // all at once: a second, nearly empty round of blocks would stream at a fraction of the bandwidth.
 template <int KIND, int MT, int NT, int D>
-constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1; }
+constexpr int stream_min_waves() { return (NT == 1 && D == 4) ? 5 : 1; }
+// Blocks of 64 rows keep nothing in LDS but the two activation buffers (32 KiB: five blocks fill the 160 KiB of a
+// compute unit exactly, and 64-row launches of 100-220 tokens are then resident at once); their row scales wait in
+// a register per thread and take over the first buffer after the k loop, and the hand-over flag sits behind them.
+template <int MT>
+constexpr bool stream_lds_overlay() { return MT >= 4; }
 
 // Hand-over between the k shares of an overflow block (their blocks run on different compute units, possibly under
 // different L2s).  The partial sums are stored and loaded with device-scope accesses, word by word (written
@@ -115,11 +120,13 @@ constexpr int stream_min_waves() { return (MT <= 2 && NT == 1 && D == 4) ? 5 : 1
 // an L2 is needed in the middle of a launch that streams through it: every wavefront stores its sums and waits until
 // the stores are acknowledged, all wavefronts meet, one thread counts in at the block's counter.  True for the
 // share that arrived last: its accumulators then hold the sums of all shares.  Nobody waits for anybody.
-template <int MT, int NBF>
+// STRIDE_MT: the tiles the kernel's largest body has; the scratch of a share is sized for that body whatever body
+// the block runs, so that the shares of different blocks never overlap.
+template <int MT, int NBF, int STRIDE_MT>
 __device__ __forceinline__ bool stream_handover(const GemmArgs& a, v4i (&acc)[MT][NBF], int over, int split, int share,
                                                 int w, int lane, int* s_last) {
   constexpr int WAVE_INTS = MT * NBF * 4 * WAVE;
-  constexpr int BLOCK_INTS = 4 * WAVE_INTS;
+  constexpr int BLOCK_INTS = 4 * STRIDE_MT * NBF * 4 * WAVE;
   int32_t* mine = a.bal_part + ((size_t)over * split + share) * BLOCK_INTS + (size_t)w * WAVE_INTS + lane;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -158,7 +165,8 @@ __device__ __forceinline__ bool stream_handover(const GemmArgs& a, v4i (&acc)[MT
 // of A is touched: a caller whose A is still being produced waits there, with its weight loads already in
 // flight.  All four wavefronts of the block must call this together (block barriers inside); when it returns
 // nobody reads the LDS buffers any more.
-template <int KIND, int MT, int NT, int D, typename BeforeA>
+// OVERLAY: the row scales live on the first activation buffer after the k loop (stream_lds_overlay of the kernel).
+template <int KIND, int MT, int NT, int D, bool OVERLAY, int STRIDE_MT, typename BeforeA>
 __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& rb, int bx, int bz, int nz, int over,
                                              int* s_last, v4i (*lds_a)[MT * 4 * WAVE], float* lds_ts, BeforeA before_a) {
   constexpr int NBF = (KIND == 1) ? 2 * NT : NT;  // B fragments per k-step
@@ -166,7 +174,9 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
   static_assert(D % 4 == 0, "D counts whole chunks");
 
   const int lane = threadIdx.x & (WAVE - 1);
-  const int w = threadIdx.x / WAVE;
+  // the wavefront's index as a scalar: its strips and their base addresses then live in scalar registers, and a
+  // weight load is a scalar base plus one lane offset that all strips share
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
   const int g = rb.group, row0 = rb.row0, nrows = rb.nrows;
   const int mt_cnt = (nrows + 15) / 16;
   const int nk64_all = a.Kdim / 64;          // k-steps of the whole reduction
@@ -192,7 +202,8 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
     }
   }
 #pragma unroll
-  for (int j = 0; j < NBF; ++j) bp[j] = wbase + ((size_t)strip[j] * nk64_all + k64_0) * 1024 + lane * 16;
+  for (int j = 0; j < NBF; ++j) bp[j] = wbase + ((size_t)strip[j] * nk64_all + k64_0) * 1024;
+  const uint32_t lane16 = lane * 16;
 
   // the first D k-steps of B are requested as soon as their addresses exist (they come from HBM and
   // take the longest); the A row lookup below overlaps with their flight
@@ -200,13 +211,16 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
   for (int s = 0; s < D; ++s)
 #pragma unroll
-    for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024));
+    for (int j = 0; j < NBF; ++j) ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)s * 1024 + lane16));
   __builtin_amdgcn_sched_barrier(0);
   before_a();
   // the activation scale of every row of the block goes to LDS now (one or two dependent loads per row, whose
   // way is then covered by the k loop instead of standing in front of the epilogue)
-  if (threadIdx.x < 16 * MT)
-    lds_ts[threadIdx.x] = ((int)threadIdx.x < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + threadIdx.x)] : 0.0f;
+  float my_ts = 0.0f;
+  if (threadIdx.x < 16 * MT) {
+    my_ts = ((int)threadIdx.x < nrows) ? a.a_scale[source_row<KIND>(a, g, row0 + threadIdx.x)] : 0.0f;
+    if constexpr (!OVERLAY) lds_ts[threadIdx.x] = my_ts;
+  }
 
   // the weight scales of this lane's output channels are requested here as well: asked for in the epilogue they
   // would cost one more round trip through a saturated memory system at the end of every block's life
@@ -222,12 +236,13 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
   // 16 half lines, and its LDS stores are conflict free (measured 0.5 us better there).
   // Rows past the end of the group alias the group's first row.
   constexpr bool WHOLE_ROWS = (KIND == 1);
-  const int8_t* arow[MT];
+  // byte offsets of the lane's pieces from a.a_q (the operand of a stream launch is far below 4 GiB: checked on the host)
+  uint32_t arow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     int rr = mt * 16 + (WHOLE_ROWS ? 4 * w + (lane >> 4) : (lane & 15));
     if (rr >= nrows) rr = 0;
-    arow[mt] = a.a_q + (size_t)source_row<KIND>(a, g, row0 + rr) * a.Kdim + (size_t)k64_0 * 64 +
+    arow[mt] = (uint32_t)source_row<KIND>(a, g, row0 + rr) * (uint32_t)a.Kdim + (uint32_t)k64_0 * 64 +
                (WHOLE_ROWS ? (lane & 15) * 16 : (lane >> 4) * 16 + w * 64);
   }
   const int a_slot = WHOLE_ROWS ? ((lane & 15) >> 2) * WAVE + (lane & 3) * 16 + 4 * w + (lane >> 4) : w * WAVE + lane;
@@ -239,42 +254,54 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
     for (int j = 0; j < NBF; ++j) acc[mt][j] = (v4i){0, 0, 0, 0};
 
   // ---- prologue: A chunk 0 -> LDS
-  v4i areg[MT];
+  // Blocks of four 16-row tiles stage the activation chunk in two halves (tiles 0-1 behind the first two k-steps
+  // of a chunk, tiles 2-3 behind the last two) through two registers' worth of loads instead of four: part of
+  // what lets the 64-row variants keep five wavefronts per SIMD.
+  constexpr int AH = (MT == 4) ? 2 : MT;   // tiles staged at a time
+  constexpr int APH = MT / AH;             // halves of a chunk's staging
+  v4i areg[AH];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt]);
+  for (int h = 0; h < APH; ++h) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) lds_a[0][mt * 4 * WAVE + a_slot] = areg[mt];
+    for (int m = 0; m < AH; ++m) areg[m] = *(const v4i*)(a.a_q + arow[h * AH + m]);
+#pragma unroll
+    for (int m = 0; m < AH; ++m) lds_a[0][(h * AH + m) * 4 * WAVE + a_slot] = areg[m];
+  }
   __syncthreads();
 
   // one chunk = 4 k-steps on ring slots [4*cc, 4*cc+4)
   auto chunk = [&](const int c, const int cc, const bool refill) {
     const int cnext = (c + 1 < nchunks) ? c + 1 : c;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) areg[mt] = *(const v4i*)(arow[mt] + (size_t)cnext * 256);
-    // keep these loads ahead of the ring refills below: they are waited for at the end of the
-    // chunk, and loads complete in order, so a later position would drain the whole ring
-    __builtin_amdgcn_sched_barrier(0);
     const v4i* la = lds_a[c & 1];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int s = cc * 4 + kk;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        v4i af = la[(mt * 4 + kk) * WAVE + lane];
-#pragma unroll
-        for (int j = 0; j < NBF; ++j) acc[mt][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, ring[s][j], acc[mt][j], 0, 0, 0);
-      }
-      // the slot is free once its MFMAs are issued: refill it with the k-step D ahead
-      if (refill) {
-#pragma unroll
-        for (int j = 0; j < NBF; ++j)
-          ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)(c * 4 + kk + D) * 1024));
-      }
-      __builtin_amdgcn_sched_barrier(0);  // one k-step at a time: refills stay spread over the chunk
-    }
     v4i* ln = lds_a[(c + 1) & 1];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) ln[mt * 4 * WAVE + a_slot] = areg[mt];
+    for (int h = 0; h < APH; ++h) {
+#pragma unroll
+      for (int m = 0; m < AH; ++m) areg[m] = *(const v4i*)(a.a_q + (arow[h * AH + m] + (uint32_t)cnext * 256));
+      // keep these loads ahead of the ring refills below: they are waited for at the end of their half of the
+      // chunk, and loads complete in order, so a later position would drain the whole ring
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kk = h * (4 / APH); kk < (h + 1) * (4 / APH); ++kk) {
+        const int s = cc * 4 + kk;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          v4i af = la[(mt * 4 + kk) * WAVE + lane];
+#pragma unroll
+          for (int j = 0; j < NBF; ++j) acc[mt][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, ring[s][j], acc[mt][j], 0, 0, 0);
+        }
+        // the slot is free once its MFMAs are issued: refill it with the k-step D ahead
+        if (refill) {
+#pragma unroll
+          for (int j = 0; j < NBF; ++j)
+            ring[s][j] = __builtin_nontemporal_load((const v4i*)(bp[j] + (size_t)(c * 4 + kk + D) * 1024 + lane16));
+        }
+        __builtin_amdgcn_sched_barrier(0);  // one k-step at a time: refills stay spread over the chunk
+      }
+      // the other buffer was last read a chunk ago, before the barrier that ended that chunk
+#pragma unroll
+      for (int m = 0; m < AH; ++m) ln[(h * AH + m) * 4 * WAVE + a_slot] = areg[m];
+    }
     __syncthreads();
   };
 
@@ -299,8 +326,13 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 #pragma unroll
   for (int cc = 0; cc < DC; ++cc) chunk(c0 + cc, cc, false);
 
+  if constexpr (OVERLAY) {
+    // the last chunk ended at a block barrier: nobody reads the activation buffers any more
+    if (threadIdx.x < 16 * MT) lds_ts[threadIdx.x] = my_ts;
+    __syncthreads();
+  }
   if (over >= 0) {
-    if (!stream_handover<MT, NBF>(a, acc, over, nz, bz, w, lane, s_last)) return;
+    if (!stream_handover<MT, NBF, STRIDE_MT>(a, acc, over, nz, bz, w, lane, s_last)) return;
   }
   // ---- epilogue
   const int col = lane & 15;
@@ -380,9 +412,19 @@ __device__ __forceinline__ void stream_block(const GemmArgs& a, const RowBlock& 
 template <int KIND, int MT, int NT, int D>
 __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void gemm_stream(GemmArgs a) {
   __shared__ v4i lds_a[2][MT * 4 * WAVE];
-  __shared__ float lds_ts[16 * MT];
-  __shared__ int s_last;
+  float* lds_ts;
+  int* s_last;
+  if constexpr (stream_lds_overlay<MT>()) {
+    lds_ts = (float*)&lds_a[0][0];
+    s_last = (int*)(lds_ts + 16 * MT);
+  } else {
+    __shared__ float ts_own[16 * MT];
+    __shared__ int last_own;
+    lds_ts = ts_own;
+    s_last = &last_own;
+  }
   RowBlock rb;
+  int bx = blockIdx.x, bz = blockIdx.z, nz = a.S, over = -1;
   if (a.bal_cus > 0) {
     // 1-d grid, balanced numbering: whole blocks, the overflow blocks' first shares, the helper shares
     const RowBlockScan sc = row_blocks_scan(a.offsets, a.G, a.extra_rows, 16 * MT);
@@ -393,12 +435,27 @@ __global__ __launch_bounds__(256, (stream_min_waves<KIND, MT, NT, D>())) void ge
     omni_host::StreamSel sel;
     if (!omni_host::stream_select(bal, n_real, (int)blockIdx.x, sel)) return;
     if (!row_blocks_find(sc, a.offsets, a.G, a.extra_rows, 16 * MT, sel.task / a.bal_cb, rb)) return;
-    stream_block<KIND, MT, NT, D>(a, rb, sel.task % a.bal_cb, sel.share, sel.over >= 0 ? bal.split : 1, sel.over, &s_last,
-                                  lds_a, lds_ts, [] {});
+    bx = sel.task % a.bal_cb;
+    bz = sel.share;
+    nz = sel.over >= 0 ? bal.split : 1;
+    over = sel.over;
+  } else if (!find_row_block(a.offsets, a.G, a.extra_rows, 16 * MT, blockIdx.y, rb)) {
     return;
   }
-  if (!find_row_block(a.offsets, a.G, a.extra_rows, 16 * MT, blockIdx.y, rb)) return;
-  stream_block<KIND, MT, NT, D>(a, rb, blockIdx.x, blockIdx.z, a.S, -1, &s_last, lds_a, lds_ts, [] {});
+  constexpr bool OVL = stream_lds_overlay<MT>();
+  if constexpr (MT == 4) {
+    // a 64-row block with at most 32 rows runs the two-tile body: half the activation loads, LDS reads and MFMAs
+    // (measured on the 64-row GEMM1: the two empty tiles cost a seventh of the launch)
+    if (rb.nrows <= 32) {
+      stream_block<KIND, 2, NT, D, OVL, MT>(a, rb, bx, bz, nz, over, s_last, (v4i(*)[2 * 4 * WAVE])lds_a, lds_ts, [] {});
+      return;
+    }
+    if (rb.nrows <= 48) {
+      stream_block<KIND, 3, NT, D, OVL, MT>(a, rb, bx, bz, nz, over, s_last, (v4i(*)[3 * 4 * WAVE])lds_a, lds_ts, [] {});
+      return;
+    }
+  }
+  stream_block<KIND, MT, NT, D, OVL, MT>(a, rb, bx, bz, nz, over, s_last, lds_a, lds_ts, [] {});
 }
 
 // Row quantisation of y = silu(gate) * up (fp32) by one wavefront: scale = max|y| / 127, q = rint(y / scale).
