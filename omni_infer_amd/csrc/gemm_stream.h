@@ -99,13 +99,14 @@ __device__ __forceinline__ void dump_acc_gemm2(const GemmArgs& a, int n, int row
 //   Requires Kdim % (64*D) == 0 (checked on the host).
 //
 // The k loop is free of data-dependent branches: rows past the end of a group read the group's
-// first row (their accumulators are never stored), every tile of the block is multiplied, and
+// first row (their accumulators are never stored), every tile of the body is multiplied (a 64-row
+// kernel picks its two-, three- or four-tile body by the block's row count before the loop), and
 // the loop is split into a part that refills the ring and a drain part, so the compiler can
 // count outstanding loads exactly and never waits for more than the oldest k-step.
 // =====================================================================================
-// Occupancy asked of the compiler: the small variants are held to 5 wavefronts per SIMD (96
-// registers) so that a decode-sized launch (about 34 row blocks x 32 channel blocks) is resident
-// all at once: a second, nearly empty round of blocks would stream at a fraction of the bandwidth.
+// Occupancy asked of the compiler: the variants with one strip (pair) per wavefront are held to 5
+// wavefronts per SIMD (96 registers) so that a launch of about 34 row blocks x 32 channel blocks is
+// resident all at once: a second, nearly empty round of blocks would stream at a fraction of the bandwidth.
 template <int KIND, int MT, int NT, int D>
 constexpr int stream_min_waves() { return (NT == 1 && D == 4) ? 5 : 1; }
 // Blocks of 64 rows keep nothing in LDS but the two activation buffers (32 KiB: five blocks fill the 160 KiB of a
