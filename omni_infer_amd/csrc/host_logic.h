@@ -227,6 +227,7 @@ OMNI_HD int stream_balance_max_helpers(int cus) { return cus > 1 ? (cus - 1) * 3
 //   OMNI_MOE_TILE_TAIL     0: tiles of the last partial round are not split along k
 //   OMNI_MOE_TILE_SPLIT    most shares of such a tile (default 4)
 //   OMNI_MOE_ROWQ          threads per row of swiglu_quant_rows
+//   OMNI_MOE_TILE_FROM      "g1,g2": expected rows per routed group above which GEMM1 / GEMM2 run the tile kernel
 //   OMNI_MOE_STREAM_BALANCE 0: the overflow blocks of a resident stream launch are not split along k
 //   OMNI_MOE_EQUAL_PROGRESS bit 0: the stream kernel of GEMM1 lowers the issue priority of its wavefronts as they
 //                          advance (default 1), bit 1: that of GEMM2 too (measured slower in every geometry)
@@ -234,6 +235,7 @@ struct Tuning {
   int force_kernel = 0, tile_wn = 4, tile_tail = 1, tile_split = 4, rowq = 0, equal_progress = 1, tile_lines = 1;
   int tile_mfma16 = 1;
   int stream_balance = 1;
+  int tile_from[3] = {0, 48, 56};  // expected rows per routed group above which GEMM1 / GEMM2 run the tile kernel
   bool have[3] = {false, false, false};
   int mt[3] = {0, 0, 0}, nt[3] = {0, 0, 0}, d[3] = {0, 0, 0}, S[3] = {0, 0, 0};
 };
@@ -266,6 +268,10 @@ inline Tuning read_tuning() {
   r.equal_progress = geti("OMNI_MOE_EQUAL_PROGRESS", 1);
   r.tile_lines = geti("OMNI_MOE_TILE_LINES", 1);
   r.stream_balance = geti("OMNI_MOE_STREAM_BALANCE", 1);
+  if (const char* e = getenv("OMNI_MOE_TILE_FROM")) {
+    int g1 = 0, g2 = 0;
+    if (sscanf(e, "%d,%d", &g1, &g2) == 2 && g1 > 0 && g2 > 0) { r.tile_from[1] = g1; r.tile_from[2] = g2; }
+  }
   for (int kind = 1; kind <= 2; ++kind) {
     const char* name = kind == 1 ? "OMNI_MOE_G1" : "OMNI_MOE_G2";
     const char* e = getenv(name);
@@ -304,12 +310,13 @@ inline Plan make_plan(int kind, int T, int K, int G, int extra_rows, int Kdim, i
   const int64_t per = (G > 0) ? avg : extra_rows;
   Plan p{};
   p.per = per;
-  // Measured on the DeepSeek-V3 shape (32 routed groups + the shared one): up to 56 expected rows per
-  // routed group the stream kernel wins (row blocks of 64 rows from 25 expected rows on, so that
-  // nearly every group is one block and its weights are read once; the shared group then takes a few
-  // blocks and re-reads its 3 % of the bytes); above that the tile kernel does.
-  p.tile = (G > 0) ? per > 56 : per > 128;
+  // Measured on the DeepSeek-V3 shape (32 routed groups + the shared one): the stream kernel wins GEMM1 up to 48
+  // expected rows per routed group and GEMM2 up to 56 (row blocks of 64 rows from 25 expected rows on, so that
+  // nearly every group is one block and its weights are read once; past 48 too many groups spill into a second
+  // block and the launch into a second round: 200 tokens 365 us against 336 us with tiles); above that the tile
+  // kernel does.
   const Tuning& tn = tuning();
+  p.tile = (G > 0) ? per > tn.tile_from[kind] : per > 128;
   const int force = tn.force_kernel;
   if (force == 1) p.tile = false;
   if (force == 2) p.tile = true;

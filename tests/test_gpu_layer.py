@@ -216,6 +216,38 @@ def test_config3_prefill_outliers_reduced(env):
     _check_out(out, out_ref)
 
 
+# ------------------------------------------------------------------ across the kernel choice
+@pytest.mark.parametrize("T,shared", [(80, True), (90, True), (100, True), (96, False), (104, False), (120, False)])
+def test_layer_across_the_kernel_crossover(env, T, shared):
+    """8 local experts, top-4 among them: T / 2 expected rows per expert.  80 tokens with the shared expert: both
+    GEMMs stream (64-row blocks whose bodies take two, three or four tiles by their row count); 90: GEMM1
+    streams, GEMM2 (whose groups count the shared rows) runs tiles; 100: both run tiles.  Without the shared expert,
+    96: both stream; 104: GEMM1 runs tiles, GEMM2 streams; 120: both tiles.  Every one against the oracle, bit exact."""
+    n_local, K, H, I = 8, 4, 1024, 512
+    names = {(80, True): ("gemm_stream", "gemm_stream"), (90, True): ("gemm_stream", "gemm_pipe"),
+             (100, True): ("gemm_pipe", "gemm_pipe"), (96, False): ("gemm_stream", "gemm_stream"),
+             (104, False): ("gemm_pipe", "gemm_stream"), (120, False): ("gemm_pipe", "gemm_pipe")}[(T, shared)]
+    M_cap = T * K + (T if shared else 0)
+    got_names = (env.ops.gemm_kernel_name(1, T, K, n_local, T if shared else 0, M_cap, H, I),
+                 env.ops.gemm_kernel_name(2, T, K, n_local, T if shared else 0, M_cap, H, I))
+    assert got_names[0].startswith(names[0]) and got_names[1].startswith(names[1]), got_names
+    lay = Layer(n_local, H, I, seed=51, shared=shared)
+    d = lay.to_device()
+    g = gen(52 + T)
+    x = tokens(T, H, 53 + T)
+    ids = torch.rand(T, n_local, generator=g).argsort(dim=1)[:, :K].to(torch.int32)
+    w = torch.rand(T, K, generator=g)
+    xq, xs = O.dynamic_quant(x)
+    out_ref = O.fused_experts_w8a8_allgather_ep(xq, xs, lay.w1_t, lay.w2_t, lay.s13, lay.s2, w, ids, (0, n_local))
+    sh = None
+    if shared:
+        out_ref = out_ref + O.shared_expert_mlp(x, *lay.shared)
+        sh = (d["sh13"], d["sh_s13"], d["sh2"], d["sh_s2"])
+    out = env.ops.moe_w8a8_layer(x.cuda(), None, w.cuda(), ids.cuda(), 0, n_local, d["w13"], d["s13"], d["w2"], d["s2"], sh,
+                                 H=H, I=I)
+    _check_out(out, out_ref)
+
+
 # ------------------------------------------------------------------ config 4: Pangu-Ultra-MoE shape
 @pytest.mark.parametrize("T", [1, 16, 128, 1024])
 def test_config4_pangu_shape(env, T):
